@@ -1,0 +1,175 @@
+/*
+ * rlx_adamw.h — C ABI of the MI355X (gfx950) AdamW + gradient-norm/clip library.
+ *
+ * Plain pointers and sizes only; every pointer named "device" is HIP device memory,
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream).  All work is
+ * stream-ordered and asynchronous unless a function says that it synchronises.  Every
+ * function returns an rlx_status; nothing here exits the process.  FP16 values are
+ * passed as uint16_t bit patterns (IEEE binary16).
+ *
+ * Each entry point names the reference interface (path inside the reference tree) that
+ * it replaces.
+ */
+#ifndef RLX_ADAMW_H
+#define RLX_ADAMW_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum {
+    RLX_OK = 0,
+    RLX_ERR_INVALID_ARG = 1,      /* null pointer, negative size, bad enum, bad plan */
+    RLX_ERR_MISALIGNED = 2,       /* pointer not aligned to its element size */
+    RLX_ERR_BAD_HYPER = 3,        /* bias correction of 0, or a non-finite hyper-parameter */
+    RLX_ERR_HIP = 4,              /* a HIP runtime call failed; see rlx_last_hip_error() */
+    RLX_ERR_NO_DEVICE = 5,
+    RLX_ERR_TOO_LARGE = 6         /* more chunks than one plan can address */
+} rlx_status;
+
+const char* rlx_status_string(int status);
+/* Text of the last HIP error seen by this thread ("" if none). */
+const char* rlx_last_hip_error(void);
+/* ABI version of the loaded library (major*100 + minor). */
+int rlx_version(void);
+
+/* ------------------------------------------------------------------------------------
+ * Operator API: one flat tensor per call.
+ * ---------------------------------------------------------------------------------- */
+
+/*
+ * Replaces launch_adamw_fp16 (include/kernels/adamw.cuh:24-39, src/kernels/adamw.cu:42-58).
+ * Same argument order and meaning: bias_correctionK = 1 - betaK^t (not the reciprocal);
+ * n <= 0 is a no-op that returns RLX_OK.  n is 64-bit.
+ * master_w may be NULL: the FP16 weight is then read as the source of truth
+ * (22 bytes per parameter instead of 28).  With a master copy model_w is write-only,
+ * as in the reference.
+ */
+int rlx_adamw_fp16(float* master_w, uint16_t* model_w, const uint16_t* grad,
+                   float* m, float* v, int64_t n,
+                   float lr, float beta1, float beta2, float eps, float weight_decay,
+                   float bias_correction1, float bias_correction2, void* stream);
+
+/* Replaces launch_adamw_fp32 (include/kernels/adamw.cuh:43-57, src/kernels/adamw.cu:93-108). */
+int rlx_adamw_fp32(float* w, const float* grad, float* m, float* v, int64_t n,
+                   float lr, float beta1, float beta2, float eps, float weight_decay,
+                   float bias_correction1, float bias_correction2, void* stream);
+
+/* Replaces fp16_to_fp32 (include/training/optimizer.h:46-57): dst[i] = (float)src[i]. */
+int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream);
+
+/* ------------------------------------------------------------------------------------
+ * Multi-tensor plan: a whole model's tensors in one launch.
+ * ---------------------------------------------------------------------------------- */
+
+enum { RLX_DTYPE_F16 = 0, RLX_DTYPE_F32 = 1 };
+
+enum {
+    RLX_TENSOR_NO_DECAY  = 1,   /* weight_decay is 0 for this tensor (embedding and norm
+                                   groups, include/training/optimizer.h:131-146) */
+    RLX_TENSOR_GRAD_ONLY = 2    /* no parameter: the buffer only takes part in the norm and
+                                   in the scale pass (the D_buf tail of the reference's
+                                   float_pool, include/training/trainer.h:330-337) */
+};
+
+typedef struct rlx_tensor_desc {
+    void*       param;    /* device; FP16 or FP32 weights [n]; NULL iff GRAD_ONLY */
+    void*       grad;     /* device; same dtype as param [n]; written only by rlx_plan_scale_grads */
+    float*      m;        /* device; first moment [n] */
+    float*      v;        /* device; second moment [n] */
+    float*      master;   /* device; FP32 master weights [n] or NULL (FP16 tensors only) */
+    int64_t     n;        /* elements, > 0 */
+    int32_t     dtype;    /* RLX_DTYPE_* */
+    uint32_t    flags;    /* RLX_TENSOR_* */
+} rlx_tensor_desc;
+
+/* Hyper-parameters of one step; the same seven floats that launch_adamw_* take. */
+typedef struct rlx_step_params {
+    float lr, beta1, beta2, eps, weight_decay;
+    float bias_correction1, bias_correction2;   /* 1 - beta^t */
+} rlx_step_params;
+
+typedef struct rlx_plan rlx_plan;
+
+/*
+ * Builds the device-resident work table for `count` tensors (the role that
+ * AdamWOptimizer::init's offset bookkeeping has, include/training/optimizer.h:188-243).
+ * Tensors are cut into chunks of `chunk_elems` elements (0 = default; otherwise a
+ * multiple of 2048); the table order is the order of `descs`, which also fixes the
+ * order of the norm reduction.  The plan borrows every pointer in `descs` and owns only
+ * its tables and the reduction workspace.  Allocates; call outside the step loop.
+ */
+int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_elems, rlx_plan** out);
+int rlx_plan_destroy(rlx_plan* plan);
+int64_t rlx_plan_num_chunks(const rlx_plan* plan);
+int64_t rlx_plan_num_elements(const rlx_plan* plan);
+int64_t rlx_plan_chunk_elems(const rlx_plan* plan);
+
+/*
+ * Global gradient L2 norm and clip scale, entirely on the device:
+ * replaces the reduce half of Trainer::clip_grad_norm_ (include/training/trainer.h:323-345,
+ * sum_sq_half_kernel / sum_sq_float_kernel :103-133).  Two passes without atomics:
+ * one FP64 partial per chunk in table order, then one block that adds the partials in
+ * a fixed order, so that the result is the same bits on every run.  Writes
+ * {sum_sq, norm = sqrtf((float)sum_sq), scale} to the plan's device result, where
+ * scale = max_norm / (norm + 1e-6f) iff norm > max_norm, else 1.0f (a NaN norm gives
+ * 1.0f, as the reference's comparison does).  No host synchronisation.
+ */
+int rlx_plan_grad_norm(rlx_plan* plan, float max_norm, void* stream);
+
+/*
+ * Copies the last result of rlx_plan_grad_norm to the host and waits for it (the
+ * blocking 4-byte copy of include/training/trainer.h:339-341).  Any out pointer may be NULL.
+ */
+int rlx_plan_norm_read(rlx_plan* plan, float* norm, float* scale, double* sum_sq, void* stream);
+
+/* Device address of the result {double sum_sq; float norm; float scale;} (16 bytes). */
+const void* rlx_plan_norm_device_ptr(const rlx_plan* plan);
+/* Device address of the per-chunk FP64 partials (rlx_plan_num_chunks values). */
+const double* rlx_plan_partials_device_ptr(const rlx_plan* plan);
+
+/*
+ * In-place scale of all gradients by the device-resident clip scale: replaces
+ * scale_half_kernel / scale_float_kernel (include/training/trainer.h:136-145,346-349).
+ * FP16 gradients are re-rounded to FP16.  A scale of exactly 1.0f leaves every bit alone.
+ */
+int rlx_plan_scale_grads(rlx_plan* plan, void* stream);
+
+/*
+ * One AdamW step over every tensor of the plan in a single launch: replaces the three
+ * launches of AdamWOptimizer::step (include/training/optimizer.h:124-146).
+ * clip_mode: RLX_CLIP_NONE  gradients are used as stored;
+ *            RLX_CLIP_FUSED the scale left by rlx_plan_grad_norm on the device is applied
+ *                           to each gradient in registers (FP16 gradients re-rounded to
+ *                           FP16 first, exactly as rlx_plan_scale_grads would have stored
+ *                           them); the gradient buffers are not written.
+ */
+enum { RLX_CLIP_NONE = 0, RLX_CLIP_FUSED = 1 };
+int rlx_plan_adamw(rlx_plan* plan, const rlx_step_params* params, int clip_mode, void* stream);
+
+/* ------------------------------------------------------------------------------------
+ * Launch tuning (process-wide; for measurement).  Unknown keys return RLX_ERR_INVALID_ARG.
+ *   "update_variant"  0..N-1   which compiled update kernel
+ *   "update_grid"     0 = one workgroup per chunk, >0 = that many persistent workgroups
+ *   "norm_grid"       same for the norm pass
+ * ---------------------------------------------------------------------------------- */
+int rlx_set_tuning(const char* key, int64_t value);
+int64_t rlx_get_tuning(const char* key);
+
+/* ------------------------------------------------------------------------------------
+ * Seeded synthetic inputs, generated on the device (no counterpart in the reference,
+ * whose gradients come from its backward pass).  value(i) = mean + std * z(seed, first+i)
+ * with z an integer-hash approximation of N(0,1); rows of row_len elements whose row
+ * hash is below zero_rows_below / 2^32 are zero.  flags: 1 = use |z|.
+ * ---------------------------------------------------------------------------------- */
+int rlx_fill_f16(uint16_t* dst, int64_t n, uint64_t seed, int64_t first, float mean, float std,
+                 uint32_t flags, int64_t row_len, uint32_t zero_rows_below, void* stream);
+int rlx_fill_f32(float* dst, int64_t n, uint64_t seed, int64_t first, float mean, float std,
+                 uint32_t flags, int64_t row_len, uint32_t zero_rows_below, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* RLX_ADAMW_H */
