@@ -96,8 +96,8 @@ typedef struct rlx_plan rlx_plan;
 /*
  * Builds the device-resident work table for `count` tensors (the role that
  * AdamWOptimizer::init's offset bookkeeping has, include/training/optimizer.h:188-243).
- * Tensors are cut into chunks of `chunk_elems` elements (0 = default; otherwise a
- * multiple of 2048); the table order is the order of `descs`, which also fixes the
+ * Tensors are cut into chunks of `chunk_elems` elements (0 = chosen from the mean tensor
+ * size; otherwise a power of two >= 2048); the table order is the order of `descs`, which also fixes the
  * order of the norm reduction.  The plan borrows every pointer in `descs` and owns only
  * its tables and the reduction workspace.  Allocates; call outside the step loop.
  */
@@ -151,9 +151,9 @@ int rlx_plan_adamw(rlx_plan* plan, const rlx_step_params* params, int clip_mode,
 
 /* ------------------------------------------------------------------------------------
  * Launch tuning (process-wide; for measurement).  Unknown keys return RLX_ERR_INVALID_ARG.
- *   "update_variant"  0..N-1   which compiled update kernel
- *   "update_grid"     0 = one workgroup per chunk, >0 = that many persistent workgroups
- *   "norm_grid"       same for the norm pass
+ *   "update_variant"  0..N-1   which compiled tile shape of the update kernel (0 = default)
+ *   "norm_grid"       0 = one workgroup per chunk, >0 = that many persistent workgroups
+ *   "norm_nt"         1 = non-temporal loads in the norm pass (default), 0 = plain
  * ---------------------------------------------------------------------------------- */
 int rlx_set_tuning(const char* key, int64_t value);
 int64_t rlx_get_tuning(const char* key);

@@ -2,10 +2,24 @@
 // C ABI declared in include/rlx_adamw.h.
 //
 // Every kernel here is a pure stream over HBM: no LDS except for the cross-wave step of
-// the norm reduction, no matrix cores.  A "chunk" is `chunk_elems` consecutive elements
-// of one tensor; a workgroup of 256 lanes (four 64-lane wavefronts) handles one chunk at
-// a time.  Inside a chunk lane t owns the 8-element groups t, t+256, t+512, ...: an FP16
-// group is one 128-bit access, an FP32 group two.
+// the norm reduction, no matrix cores.
+//
+// Work is described by one 64-byte record per "chunk" (`chunk_elems` consecutive elements
+// of one tensor) holding the chunk's resolved pointers, so that a workgroup needs a single
+// scalar load to find its operands.
+//
+// Update kernel: a chunk is cut into tiles of 256 elements and every tile is one small
+// workgroup (128 lanes, two elements per lane: one 32-bit access per FP16 stream and one
+// 64-bit access per FP32 stream, each instruction contiguous across the wavefront, all
+// marked non-temporal).  On MI355X this shape measured ~6.7 TB/s on the seven streams of
+// the update against ~5.3 TB/s for 128-bit accesses with several KB per workgroup: what
+// matters for a mixed read/write stream is that the set of addresses in flight stays a
+// narrow window, which many tiny workgroups dispatched in order give and fat workgroups or
+// grid-stride loops do not.  Consecutive workgroups go round-robin to the 8 XCDs; an optional
+// swizzle (K > 1) hands each XCD K neighbouring tiles, which did not pay in measurements.
+//
+// Norm kernel: one workgroup of 256 lanes per chunk with 128-bit reads; one FP64 partial
+// per chunk in a fixed slot, then a single-workgroup pass in fixed order (no atomics).
 //
 // Arithmetic follows src/kernels/adamw.cu:25-39 of the reference operation by operation
 // and is compiled without FMA contraction, with IEEE division and square root and with
@@ -24,33 +38,33 @@
 
 namespace {
 
-constexpr int kBlock = 256;                   // lanes per workgroup
-constexpr int kVec = 8;                       // elements per lane per group
-constexpr int kGroup = kBlock * kVec;         // 2048 elements per workgroup-wide group
-constexpr int64_t kDefaultChunk = 8192;
+constexpr int kNormBlock = 256;               // lanes per workgroup of the norm and scale passes
+constexpr int kVec = 8;                       // elements per lane per group there
+constexpr int kGroup = kNormBlock * kVec;     // 2048
+constexpr int64_t kMinChunk = 2048;
+constexpr int64_t kBigChunk = 8192;
 constexpr int kFinalBlock = 1024;
 
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
-struct DevTensor {
+// One chunk of one tensor, pointers already advanced to the chunk's first element.
+struct ChunkRec {
     void* p;
     void* g;
     float* m;
     float* v;
     float* master;
-    int64_t n;
-    int32_t dtype;
-    uint32_t flags;      // RLX_TENSOR_* | kAligned
-    int64_t pad;
+    uint32_t count;      // elements in this chunk (the last chunk of a tensor may be short)
+    uint32_t flags;      // RLX_TENSOR_* | kF32 | valign << kValignShift
+    int64_t pad[2];
 };
-static_assert(sizeof(DevTensor) == 64, "DevTensor is one 64-byte record");
-constexpr uint32_t kAligned = 0x100;          // every pointer of the tensor is 16-byte aligned
-
-struct DevChunk {
-    int32_t tensor;
-    int32_t index;       // chunk number inside the tensor
-};
+static_assert(sizeof(ChunkRec) == 64, "ChunkRec is one 64-byte record");
+constexpr uint32_t kF32 = 0x10;               // FP32 parameter and gradient
+constexpr int kValignShift = 8;               // flags bits 8..11: widest lane vector (1,2,4,8 elements)
+                                              // for which every stream of the chunk is aligned
 
 struct NormResult {
     double sum_sq;
@@ -74,8 +88,8 @@ __device__ __forceinline__ uint32_t f2h(float x) {
     return (uint32_t)__builtin_bit_cast(uint16_t, (_Float16)x);     // round to nearest even
 }
 
-// Every buffer handed to this library is HIP device memory, so all vector accesses go
-// through global-address-space pointers (global_load/global_store rather than flat).
+// Every buffer handed to this library is HIP device memory, so all accesses go through
+// global-address-space pointers (global_load/global_store rather than flat).
 #define RLX_GLOBAL __attribute__((address_space(1)))
 
 template <bool NT, typename T>
@@ -106,242 +120,201 @@ __device__ __forceinline__ void adamw_elem(float g, float& m, float& v, float& w
 // Clip as a preceding scale pass would have stored it (trainer.h:136-139): re-round to FP16.
 __device__ __forceinline__ float clip_f16(float g, float scale) { return h2f(f2h(g * scale)); }
 
-struct Group16 {          // eight FP16 parameters with their state, in registers
-    u32x4 p, g;
-    f32x4 m0, m1, v0, v1, w0, w1;
-};
+// E packed FP16 values and E FP32 values as one access each.
+template <int E> struct Lane;
+template <> struct Lane<1> { typedef uint16_t H; typedef float F; };
+template <> struct Lane<2> { typedef uint32_t H; typedef f32x2 F; };
+template <> struct Lane<4> { typedef u32x2 H; typedef f32x4 F; };
 
-template <bool NT>
-__device__ __forceinline__ void load_group16(Group16& r, const DevTensor& t, int64_t elem, bool has_master) {
-    r.g = ldg<NT>((const u32x4*)((const uint16_t*)t.g + elem));
-    r.m0 = ldg<NT>((const f32x4*)(t.m + elem));
-    r.m1 = ldg<NT>((const f32x4*)(t.m + elem) + 1);
-    r.v0 = ldg<NT>((const f32x4*)(t.v + elem));
-    r.v1 = ldg<NT>((const f32x4*)(t.v + elem) + 1);
-    if (has_master) {
-        r.w0 = ldg<NT>((const f32x4*)(t.master + elem));
-        r.w1 = ldg<NT>((const f32x4*)(t.master + elem) + 1);
-    } else {
-        r.p = ldg<NT>((const u32x4*)((const uint16_t*)t.p + elem));
+template <int E>
+__device__ __forceinline__ void unpack_h(typename Lane<E>::H x, float* out) {
+    if constexpr (E == 1) out[0] = h2f(x);
+    else if constexpr (E == 2) { out[0] = h2f(x & 0xFFFFu); out[1] = h2f(x >> 16); }
+    else { out[0] = h2f(x[0] & 0xFFFFu); out[1] = h2f(x[0] >> 16); out[2] = h2f(x[1] & 0xFFFFu); out[3] = h2f(x[1] >> 16); }
+}
+
+template <int E>
+__device__ __forceinline__ typename Lane<E>::H pack_h(const float* w) {
+    if constexpr (E == 1) return (uint16_t)f2h(w[0]);
+    else if constexpr (E == 2) return f2h(w[0]) | (f2h(w[1]) << 16);
+    else { u32x2 o; o[0] = f2h(w[0]) | (f2h(w[1]) << 16); o[1] = f2h(w[2]) | (f2h(w[3]) << 16); return o; }
+}
+
+template <int E>
+__device__ __forceinline__ void unpack_f(typename Lane<E>::F x, float* out) {
+    if constexpr (E == 1) out[0] = x;
+    else {
+#pragma unroll
+        for (int k = 0; k < E; k++) out[k] = x[k];
     }
 }
 
-template <bool NT>
-__device__ __forceinline__ void finish_group16(Group16& r, const DevTensor& t, int64_t elem, bool has_master,
-                                               const Hyper& h, float wd, float scale, bool clip) {
-    float g[8], m[8], v[8], w[8];
+template <int E>
+__device__ __forceinline__ typename Lane<E>::F pack_f(const float* x) {
+    if constexpr (E == 1) return x[0];
+    else {
+        typename Lane<E>::F o;
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-        g[2 * k] = h2f(r.g[k] & 0xFFFFu);
-        g[2 * k + 1] = h2f(r.g[k] >> 16);
-        m[k] = r.m0[k]; m[4 + k] = r.m1[k];
-        v[k] = r.v0[k]; v[4 + k] = r.v1[k];
+        for (int k = 0; k < E; k++) o[k] = x[k];
+        return o;
     }
-    if (has_master) {
-#pragma unroll
-        for (int k = 0; k < 4; k++) { w[k] = r.w0[k]; w[4 + k] = r.w1[k]; }
-    } else {
-#pragma unroll
-        for (int k = 0; k < 4; k++) { w[2 * k] = h2f(r.p[k] & 0xFFFFu); w[2 * k + 1] = h2f(r.p[k] >> 16); }
-    }
-    if (clip) {
-#pragma unroll
-        for (int k = 0; k < 8; k++) g[k] = clip_f16(g[k], scale);
-    }
-#pragma unroll
-    for (int k = 0; k < 8; k++) adamw_elem(g[k], m[k], v[k], w[k], h, wd);
-    f32x4 a, b;
-#pragma unroll
-    for (int k = 0; k < 4; k++) { a[k] = m[k]; b[k] = m[4 + k]; }
-    stg<NT>((f32x4*)(t.m + elem), a);
-    stg<NT>((f32x4*)(t.m + elem) + 1, b);
-#pragma unroll
-    for (int k = 0; k < 4; k++) { a[k] = v[k]; b[k] = v[4 + k]; }
-    stg<NT>((f32x4*)(t.v + elem), a);
-    stg<NT>((f32x4*)(t.v + elem) + 1, b);
-    if (has_master) {
-#pragma unroll
-        for (int k = 0; k < 4; k++) { a[k] = w[k]; b[k] = w[4 + k]; }
-        stg<NT>((f32x4*)(t.master + elem), a);
-        stg<NT>((f32x4*)(t.master + elem) + 1, b);
-    }
-    u32x4 out;
-#pragma unroll
-    for (int k = 0; k < 4; k++) out[k] = f2h(w[2 * k]) | (f2h(w[2 * k + 1]) << 16);
-    stg<NT>((u32x4*)((uint16_t*)t.p + elem), out);
 }
 
-// Scalar path: unaligned tensors and the last, partial group of a tensor.
-__device__ __forceinline__ void update_scalar16(const DevTensor& t, int64_t i, const Hyper& h, float wd,
+// Element-by-element path: chunks whose streams are not aligned for the lane vector, and the
+// last, partial vector of a tensor.
+__device__ __forceinline__ void update_scalar16(const ChunkRec& r, int64_t i, const Hyper& h, float wd,
                                                 float scale, bool clip) {
-    uint16_t* p = (uint16_t*)t.p;
-    float g = h2f(((const uint16_t*)t.g)[i]);
+    uint16_t* p = (uint16_t*)r.p + i;
+    float g = h2f(ldg<true>((const uint16_t*)r.g + i));
     if (clip) g = clip_f16(g, scale);
-    float m = t.m[i], v = t.v[i];
-    float w = t.master ? t.master[i] : h2f(p[i]);
+    float m = ldg<true>(r.m + i), v = ldg<true>(r.v + i);
+    float w = r.master ? ldg<true>(r.master + i) : h2f(ldg<true>(p));
     adamw_elem(g, m, v, w, h, wd);
-    t.m[i] = m;
-    t.v[i] = v;
-    if (t.master) t.master[i] = w;
-    p[i] = (uint16_t)f2h(w);
+    stg<true>(r.m + i, m);
+    stg<true>(r.v + i, v);
+    if (r.master) stg<true>(r.master + i, w);
+    stg<true>(p, (uint16_t)f2h(w));
 }
 
-__device__ __forceinline__ void update_scalar32(const DevTensor& t, int64_t i, const Hyper& h, float wd,
+__device__ __forceinline__ void update_scalar32(const ChunkRec& r, int64_t i, const Hyper& h, float wd,
                                                 float scale, bool clip) {
-    float* p = (float*)t.p;
-    float g = ((const float*)t.g)[i];
+    float* p = (float*)r.p + i;
+    float g = ldg<true>((const float*)r.g + i);
     if (clip) g = g * scale;                    // scale_float_kernel, trainer.h:142-145
-    float m = t.m[i], v = t.v[i], w = p[i];
+    float m = ldg<true>(r.m + i), v = ldg<true>(r.v + i), w = ldg<true>(p);
     adamw_elem(g, m, v, w, h, wd);
-    t.m[i] = m;
-    t.v[i] = v;
-    p[i] = w;
-}
-
-// Eight FP32 parameters (norm weights): the same update, in place (adamw.cu:80-90).
-template <bool NT>
-__device__ __forceinline__ void update_group32(const DevTensor& t, int64_t elem, const Hyper& h, float wd,
-                                               float scale, bool clip) {
-    f32x4 pw[2], gw[2], mw[2], vw[2];
-#pragma unroll
-    for (int q = 0; q < 2; q++) {
-        pw[q] = ldg<NT>((const f32x4*)((const float*)t.p + elem) + q);
-        gw[q] = ldg<NT>((const f32x4*)((const float*)t.g + elem) + q);
-        mw[q] = ldg<NT>((const f32x4*)(t.m + elem) + q);
-        vw[q] = ldg<NT>((const f32x4*)(t.v + elem) + q);
-    }
-#pragma unroll
-    for (int q = 0; q < 2; q++) {
-#pragma unroll
-        for (int k = 0; k < 4; k++) {
-            float g = gw[q][k];
-            if (clip) g = g * scale;
-            float m = mw[q][k], v = vw[q][k], w = pw[q][k];
-            adamw_elem(g, m, v, w, h, wd);
-            mw[q][k] = m; vw[q][k] = v; pw[q][k] = w;
-        }
-        stg<NT>((f32x4*)(t.m + elem) + q, mw[q]);
-        stg<NT>((f32x4*)(t.v + elem) + q, vw[q]);
-        stg<NT>((f32x4*)((float*)t.p + elem) + q, pw[q]);
-    }
+    stg<true>(r.m + i, m);
+    stg<true>(r.v + i, v);
+    stg<true>(p, w);
 }
 
 // ---------------------------------------------------------------------------------------
-// Update kernel.  U = groups per lane whose loads are all issued before the first use.
-// SINGLE: one tensor passed by value (the operator API); otherwise the plan's tables.
+// Update kernel: one workgroup of BLOCK lanes per tile of E*BLOCK elements.
+// K > 1: workgroups b, b+8, ... land on the same XCD; groups of 8*K tiles are permuted so
+// that each XCD gets K neighbouring tiles.
+// SINGLE: one flat tensor passed by value (the operator API); otherwise the plan's records.
 // ---------------------------------------------------------------------------------------
 
-template <int U, bool NT, bool SINGLE>
-__global__ __launch_bounds__(kBlock) void adamw_update_kernel(
-    const DevTensor* __restrict__ tensors, const DevChunk* __restrict__ chunks, DevTensor single,
-    int64_t n_chunks, int64_t chunk_elems, Hyper h, const NormResult* __restrict__ norm)
+template <int E, int BLOCK, int K, bool SINGLE>
+__global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
+    const ChunkRec* __restrict__ recs, ChunkRec single, int64_t single_n, int64_t first_tile, int64_t n_tiles,
+    int tiles_per_chunk_log2, Hyper h, const NormResult* __restrict__ norm)
 {
-    const int tid = threadIdx.x;
+    constexpr int TILE = E * BLOCK;
+    int64_t b = blockIdx.x;
+    if constexpr (K > 1) {
+        const int64_t grp = b / (8 * K), r = b % (8 * K);
+        b = grp * (8 * K) + (r % 8) * K + (r / 8);
+    }
+    const int64_t tile = first_tile + b;
+    if (tile >= n_tiles) return;
+
+    ChunkRec r;
+    int64_t off;         // first element of the tile, relative to r's pointers
+    int64_t left;        // elements from there to the end of the chunk / tensor
+    if constexpr (SINGLE) {
+        r = single;
+        off = tile * TILE;
+        left = single_n - off;
+    } else {
+        r = recs[tile >> tiles_per_chunk_log2];
+        off = (tile & ((1 << tiles_per_chunk_log2) - 1)) * TILE;
+        left = (int64_t)r.count - off;
+    }
+    if (left <= 0 || (r.flags & RLX_TENSOR_GRAD_ONLY)) return;
+    const int n_here = left < TILE ? (int)left : TILE;
     const bool clip = norm != nullptr;
     const float scale = clip ? norm->scale : 1.0f;
+    const float wd = (r.flags & RLX_TENSOR_NO_DECAY) ? 0.0f : h.weight_decay;
+    const bool is_f32 = (r.flags & kF32) != 0;
+    const int valign = (r.flags >> kValignShift) & 0xF;
+    const int e0 = threadIdx.x * E;
+    const int64_t i0 = off + e0;
 
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        DevTensor t;
-        int64_t start;
-        if constexpr (SINGLE) {
-            t = single;
-            start = c * chunk_elems;
-        } else {
-            DevChunk ch = chunks[c];
-            t = tensors[ch.tensor];
-            start = (int64_t)ch.index * chunk_elems;
+    if (valign < E || e0 + E > n_here) {
+        for (int e = e0; e < e0 + E && e < n_here; e++) {
+            if (is_f32) update_scalar32(r, off + e, h, wd, scale, clip);
+            else update_scalar16(r, off + e, h, wd, scale, clip);
         }
-        if (t.flags & RLX_TENSOR_GRAD_ONLY) continue;
-        const float wd = (t.flags & RLX_TENSOR_NO_DECAY) ? 0.0f : h.weight_decay;
-        const int64_t left = t.n - start;
-        const int64_t count = left < chunk_elems ? left : chunk_elems;
-        const bool aligned = (t.flags & kAligned) != 0;
+        return;
+    }
 
-        if (!aligned) {
-            for (int64_t i = start + tid; i < start + count; i += kBlock) {
-                if (t.dtype == RLX_DTYPE_F16) update_scalar16(t, i, h, wd, scale, clip);
-                else update_scalar32(t, i, h, wd, scale, clip);
-            }
-            continue;
-        }
-
-        if (t.dtype == RLX_DTYPE_F16) {
-            const bool has_master = t.master != nullptr;
-            int64_t done = 0;
-            // full tiles of U groups: every load of the tile is in flight before any use
-            for (; done + (int64_t)U * kGroup <= count; done += (int64_t)U * kGroup) {
-                Group16 r[U];
+    typedef typename Lane<E>::H HV;
+    typedef typename Lane<E>::F FV;
+    float g[E], m[E], v[E], w[E];
+    if (!is_f32) {
+        const bool has_master = r.master != nullptr;
+        const HV gw = ldg<true>((const HV*)((const uint16_t*)r.g + i0));
+        const FV mw = ldg<true>((const FV*)(r.m + i0));
+        const FV vw = ldg<true>((const FV*)(r.v + i0));
+        if (has_master) unpack_f<E>(ldg<true>((const FV*)(r.master + i0)), w);
+        else unpack_h<E>(ldg<true>((const HV*)((const uint16_t*)r.p + i0)), w);
+        unpack_h<E>(gw, g);
+        unpack_f<E>(mw, m);
+        unpack_f<E>(vw, v);
+        if (clip) {
 #pragma unroll
-                for (int j = 0; j < U; j++)
-                    load_group16<NT>(r[j], t, start + done + (int64_t)(j * kBlock + tid) * kVec, has_master);
-#pragma unroll
-                for (int j = 0; j < U; j++)
-                    finish_group16<NT>(r[j], t, start + done + (int64_t)(j * kBlock + tid) * kVec, has_master,
-                                       h, wd, scale, clip);
-            }
-            // remaining whole groups, then the last partial group element by element
-            for (; done < count; done += kGroup) {
-                const int64_t off = done + (int64_t)tid * kVec;
-                if (off + kVec <= count) {
-                    Group16 r;
-                    load_group16<NT>(r, t, start + off, has_master);
-                    finish_group16<NT>(r, t, start + off, has_master, h, wd, scale, clip);
-                } else {
-                    for (int64_t i = off; i < count; i++) update_scalar16(t, start + i, h, wd, scale, clip);
-                }
-            }
-        } else {
-            for (int64_t done = 0; done < count; done += kGroup) {
-                const int64_t off = done + (int64_t)tid * kVec;
-                if (off + kVec <= count) {
-                    update_group32<NT>(t, start + off, h, wd, scale, clip);
-                } else {
-                    for (int64_t i = off; i < count; i++) update_scalar32(t, start + i, h, wd, scale, clip);
-                }
-            }
+            for (int k = 0; k < E; k++) g[k] = clip_f16(g[k], scale);
         }
+#pragma unroll
+        for (int k = 0; k < E; k++) adamw_elem(g[k], m[k], v[k], w[k], h, wd);
+        stg<true>((FV*)(r.m + i0), pack_f<E>(m));
+        stg<true>((FV*)(r.v + i0), pack_f<E>(v));
+        if (has_master) stg<true>((FV*)(r.master + i0), pack_f<E>(w));
+        stg<true>((HV*)((uint16_t*)r.p + i0), pack_h<E>(w));
+    } else {
+        // FP32 parameters (norm weights): the same update, in place (adamw.cu:80-90)
+        unpack_f<E>(ldg<true>((const FV*)((const float*)r.g + i0)), g);
+        unpack_f<E>(ldg<true>((const FV*)(r.m + i0)), m);
+        unpack_f<E>(ldg<true>((const FV*)(r.v + i0)), v);
+        unpack_f<E>(ldg<true>((const FV*)((const float*)r.p + i0)), w);
+        if (clip) {
+#pragma unroll
+            for (int k = 0; k < E; k++) g[k] = g[k] * scale;
+        }
+#pragma unroll
+        for (int k = 0; k < E; k++) adamw_elem(g[k], m[k], v[k], w[k], h, wd);
+        stg<true>((FV*)(r.m + i0), pack_f<E>(m));
+        stg<true>((FV*)(r.v + i0), pack_f<E>(v));
+        stg<true>((FV*)((float*)r.p + i0), pack_f<E>(w));
     }
 }
 
 // ---------------------------------------------------------------------------------------
-// Norm pass 1: one FP64 partial per chunk, written to the chunk's own slot.
+// Norm pass 1: one workgroup per chunk, one FP64 partial per chunk in the chunk's own slot.
 // Order inside a chunk (restated on the CPU by the test oracle): lane t adds x*x of its
-// groups t, t+256, ... element by element into one FP32 accumulator; the 64 lanes of a
-// wavefront combine by xor butterfly with masks 32,16,8,4,2,1; the four wavefront sums
-// go through LDS and are added in FP64 in wavefront order.
+// 8-element groups t, t+256, ... element by element into one FP32 accumulator; the 64
+// lanes of a wavefront combine by xor butterfly with masks 32,16,8,4,2,1; the four
+// wavefront sums go through LDS and are added in FP64 in wavefront order.
 // ---------------------------------------------------------------------------------------
 
 template <bool NT>
-__global__ __launch_bounds__(kBlock) void sumsq_partials_kernel(
-    const DevTensor* __restrict__ tensors, const DevChunk* __restrict__ chunks,
-    int64_t n_chunks, int64_t chunk_elems, double* __restrict__ partials)
+__global__ __launch_bounds__(kNormBlock) void sumsq_partials_kernel(
+    const ChunkRec* __restrict__ recs, int64_t n_chunks, double* __restrict__ partials)
 {
-    __shared__ float wave_sum[kBlock / 64];
+    __shared__ float wave_sum[kNormBlock / 64];
     const int tid = threadIdx.x;
 
     for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const DevChunk ch = chunks[c];
-        const DevTensor t = tensors[ch.tensor];
-        const int64_t start = (int64_t)ch.index * chunk_elems;
-        const int64_t left = t.n - start;
-        const int64_t count = left < chunk_elems ? left : chunk_elems;
-        const bool aligned = (t.flags & kAligned) != 0;
+        const ChunkRec r = recs[c];
+        const int64_t count = r.count;
+        const bool aligned = ((r.flags >> kValignShift) & 0xF) >= 8;
 
         float acc = 0.0f;
-        if (t.dtype == RLX_DTYPE_F16) {
-            const uint16_t* g = (const uint16_t*)t.g + start;
+        if (!(r.flags & kF32)) {
+            const uint16_t* g = (const uint16_t*)r.g;
             int64_t done = 0;
             if (aligned) {
                 for (; done + 4 * (int64_t)kGroup <= count; done += 4 * (int64_t)kGroup) {
-                    u32x4 r[4];
+                    u32x4 x[4];
 #pragma unroll
                     for (int j = 0; j < 4; j++)
-                        r[j] = ldg<NT>((const u32x4*)(g + done + (int64_t)(j * kBlock + tid) * kVec));
+                        x[j] = ldg<NT>((const u32x4*)(g + done + (int64_t)(j * kNormBlock + tid) * kVec));
 #pragma unroll
                     for (int j = 0; j < 4; j++) {
 #pragma unroll
                         for (int k = 0; k < 4; k++) {
-                            float a = h2f(r[j][k] & 0xFFFFu), b = h2f(r[j][k] >> 16);
+                            float a = h2f(x[j][k] & 0xFFFFu), b = h2f(x[j][k] >> 16);
                             acc = acc + a * a;
                             acc = acc + b * b;
                         }
@@ -351,32 +324,35 @@ __global__ __launch_bounds__(kBlock) void sumsq_partials_kernel(
             for (; done < count; done += kGroup) {
                 const int64_t off = done + (int64_t)tid * kVec;
                 if (aligned && off + kVec <= count) {
-                    u32x4 r = ldg<NT>((const u32x4*)(g + off));
+                    u32x4 x = ldg<NT>((const u32x4*)(g + off));
 #pragma unroll
                     for (int k = 0; k < 4; k++) {
-                        float a = h2f(r[k] & 0xFFFFu), b = h2f(r[k] >> 16);
+                        float a = h2f(x[k] & 0xFFFFu), b = h2f(x[k] >> 16);
                         acc = acc + a * a;
                         acc = acc + b * b;
                     }
                 } else {
                     for (int64_t i = off; i < off + kVec && i < count; i++) {
-                        float a = h2f(g[i]);
+                        float a = h2f(ldg<NT>(g + i));
                         acc = acc + a * a;
                     }
                 }
             }
         } else {
-            const float* g = (const float*)t.g + start;
+            const float* g = (const float*)r.g;
             for (int64_t done = 0; done < count; done += kGroup) {
                 const int64_t off = done + (int64_t)tid * kVec;
                 if (aligned && off + kVec <= count) {
-                    f32x4 r0 = ldg<NT>((const f32x4*)(g + off)), r1 = ldg<NT>((const f32x4*)(g + off) + 1);
+                    f32x4 x0 = ldg<NT>((const f32x4*)(g + off)), x1 = ldg<NT>((const f32x4*)(g + off) + 1);
 #pragma unroll
-                    for (int k = 0; k < 4; k++) acc = acc + r0[k] * r0[k];
+                    for (int k = 0; k < 4; k++) acc = acc + x0[k] * x0[k];
 #pragma unroll
-                    for (int k = 0; k < 4; k++) acc = acc + r1[k] * r1[k];
+                    for (int k = 0; k < 4; k++) acc = acc + x1[k] * x1[k];
                 } else {
-                    for (int64_t i = off; i < off + kVec && i < count; i++) acc = acc + g[i] * g[i];
+                    for (int64_t i = off; i < off + kVec && i < count; i++) {
+                        float a = ldg<NT>(g + i);
+                        acc = acc + a * a;
+                    }
                 }
             }
         }
@@ -388,7 +364,7 @@ __global__ __launch_bounds__(kBlock) void sumsq_partials_kernel(
         if (tid == 0) {
             double total = 0.0;
 #pragma unroll
-            for (int w = 0; w < kBlock / 64; w++) total += (double)wave_sum[w];
+            for (int w = 0; w < kNormBlock / 64; w++) total += (double)wave_sum[w];
             partials[c] = total;
         }
         __syncthreads();
@@ -423,38 +399,33 @@ __global__ __launch_bounds__(kFinalBlock) void sumsq_final_kernel(
 }
 
 // In-place scale of the gradients (trainer.h:136-145).  Exactly 1.0f: nothing is touched.
-template <bool NT>
-__global__ __launch_bounds__(kBlock) void scale_grads_kernel(
-    const DevTensor* __restrict__ tensors, const DevChunk* __restrict__ chunks,
-    int64_t n_chunks, int64_t chunk_elems, const NormResult* __restrict__ norm)
+__global__ __launch_bounds__(kNormBlock) void scale_grads_kernel(
+    const ChunkRec* __restrict__ recs, int64_t n_chunks, const NormResult* __restrict__ norm)
 {
     const float scale = norm->scale;
     if (scale == 1.0f) return;
     const int tid = threadIdx.x;
     for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const DevChunk ch = chunks[c];
-        const DevTensor t = tensors[ch.tensor];
-        const int64_t start = (int64_t)ch.index * chunk_elems;
-        const int64_t left = t.n - start;
-        const int64_t count = left < chunk_elems ? left : chunk_elems;
-        const bool aligned = (t.flags & kAligned) != 0;
-        if (t.dtype == RLX_DTYPE_F16) {
-            uint16_t* g = (uint16_t*)t.g + start;
+        const ChunkRec r = recs[c];
+        const int64_t count = r.count;
+        const bool aligned = ((r.flags >> kValignShift) & 0xF) >= 8;
+        if (!(r.flags & kF32)) {
+            uint16_t* g = (uint16_t*)r.g;
             for (int64_t done = 0; done < count; done += kGroup) {
                 const int64_t off = done + (int64_t)tid * kVec;
                 if (aligned && off + kVec <= count) {
-                    u32x4 r = ldg<NT>((const u32x4*)(g + off));
+                    u32x4 x = ldg<true>((const u32x4*)(g + off));
 #pragma unroll
                     for (int k = 0; k < 4; k++)
-                        r[k] = f2h(h2f(r[k] & 0xFFFFu) * scale) | (f2h(h2f(r[k] >> 16) * scale) << 16);
-                    stg<NT>((u32x4*)(g + off), r);
+                        x[k] = f2h(h2f(x[k] & 0xFFFFu) * scale) | (f2h(h2f(x[k] >> 16) * scale) << 16);
+                    stg<true>((u32x4*)(g + off), x);
                 } else {
                     for (int64_t i = off; i < off + kVec && i < count; i++)
                         g[i] = (uint16_t)f2h(h2f(g[i]) * scale);
                 }
             }
         } else {
-            float* g = (float*)t.g + start;
+            float* g = (float*)r.g;
             for (int64_t done = 0; done < count; done += kGroup) {
                 const int64_t off = done + (int64_t)tid * kVec;
                 for (int64_t i = off; i < off + kVec && i < count; i++) g[i] = g[i] * scale;
@@ -463,10 +434,10 @@ __global__ __launch_bounds__(kBlock) void scale_grads_kernel(
     }
 }
 
-__global__ __launch_bounds__(kBlock) void fp16_to_fp32_kernel(float* __restrict__ dst,
-                                                              const uint16_t* __restrict__ src, int64_t n)
+__global__ __launch_bounds__(256) void fp16_to_fp32_kernel(float* __restrict__ dst,
+                                                           const uint16_t* __restrict__ src, int64_t n)
 {
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock)
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
         dst[i] = h2f(src[i]);
 }
 
@@ -474,6 +445,8 @@ __global__ __launch_bounds__(kBlock) void fp16_to_fp32_kernel(float* __restrict_
 // Seeded synthetic inputs: integer hash -> sum of eight 16-bit uniforms -> one FP32
 // multiply and one FP32 add, so that a host restatement gives the same bits without libm.
 // ---------------------------------------------------------------------------------------
+
+constexpr int kFillBlock = 256;
 
 __host__ __device__ inline uint64_t hash64(uint64_t seed, uint64_t idx) {
     uint64_t z = seed + idx * 0x9E3779B97F4A7C15ULL;
@@ -502,11 +475,11 @@ __device__ inline float fill_value(uint64_t seed, uint64_t i, float mean, float 
 }
 
 template <typename T>
-__global__ __launch_bounds__(kBlock) void fill_kernel(T* __restrict__ dst, int64_t n, uint64_t seed, int64_t first,
+__global__ __launch_bounds__(kFillBlock) void fill_kernel(T* __restrict__ dst, int64_t n, uint64_t seed, int64_t first,
                                                       float mean, float std, uint32_t flags, int64_t row_len,
                                                       uint32_t zero_rows_below)
 {
-    for (int64_t i = (int64_t)blockIdx.x * kBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kBlock) {
+    for (int64_t i = (int64_t)blockIdx.x * kFillBlock + threadIdx.x; i < n; i += (int64_t)gridDim.x * kFillBlock) {
         const float x = fill_value(seed, (uint64_t)(first + i), mean, std, flags, row_len, zero_rows_below);
         if constexpr (sizeof(T) == 2) dst[i] = (uint16_t)f2h(x);
         else dst[i] = x;
@@ -532,19 +505,13 @@ int hip_fail(hipError_t e, const char* what) {
 
 struct Tuning {
     int64_t update_variant = 0;
-    int64_t update_grid = 0;
     int64_t norm_grid = 0;
-    int64_t norm_nt = 0;
+    int64_t norm_nt = 1;
 } g_tuning;
 
-constexpr int64_t kMaxGrid = 1 << 22;     // grid * 256 lanes stays below 2^32
-
-inline int64_t pick_grid(int64_t n_chunks, int64_t tuned) {
-    int64_t g = tuned > 0 ? tuned : n_chunks;
-    if (g > n_chunks) g = n_chunks;
-    if (g > kMaxGrid) g = kMaxGrid;
-    return g < 1 ? 1 : g;
-}
+constexpr int kNumUpdateVariants = 8;
+constexpr int64_t kMaxTilesPerLaunch = 1 << 23;   // workgroups per launch; times 256 lanes stays below 2^32
+constexpr int64_t kMaxNormGrid = 1 << 22;
 
 inline bool is_aligned(const void* p, size_t a) { return ((uintptr_t)p & (a - 1)) == 0; }
 
@@ -564,8 +531,7 @@ Hyper make_hyper(float lr, float beta1, float beta2, float eps, float wd, float 
     return h;
 }
 
-// Fills the derived fields of a device record; returns a status for bad descriptors.
-int make_dev_tensor(const rlx_tensor_desc& d, DevTensor& t) {
+int check_desc(const rlx_tensor_desc& d) {
     if (d.n <= 0 || !d.grad) return RLX_ERR_INVALID_ARG;
     if (d.dtype != RLX_DTYPE_F16 && d.dtype != RLX_DTYPE_F32) return RLX_ERR_INVALID_ARG;
     if (d.flags & ~(uint32_t)(RLX_TENSOR_NO_DECAY | RLX_TENSOR_GRAD_ONLY)) return RLX_ERR_INVALID_ARG;
@@ -576,26 +542,68 @@ int make_dev_tensor(const rlx_tensor_desc& d, DevTensor& t) {
     if (!is_aligned(d.grad, es) || !is_aligned(d.param, es) || !is_aligned(d.m, 4) || !is_aligned(d.v, 4) ||
         !is_aligned(d.master, 4))
         return RLX_ERR_MISALIGNED;
-    t.p = d.param; t.g = d.grad; t.m = d.m; t.v = d.v; t.master = d.master;
-    t.n = d.n; t.dtype = d.dtype; t.flags = d.flags; t.pad = 0;
-    if (is_aligned(d.grad, 16) && is_aligned(d.param, 16) && is_aligned(d.m, 16) && is_aligned(d.v, 16) &&
-        is_aligned(d.master, 16))
-        t.flags |= kAligned;
     return RLX_OK;
 }
 
+// Record of the chunk that starts `start` elements into the tensor.
+ChunkRec make_rec(const rlx_tensor_desc& d, int64_t start, int64_t count) {
+    const size_t es = d.dtype == RLX_DTYPE_F16 ? 2 : 4;
+    ChunkRec r;
+    r.p = d.param ? (char*)d.param + start * es : nullptr;
+    r.g = (char*)d.grad + start * es;
+    r.m = d.m ? d.m + start : nullptr;
+    r.v = d.v ? d.v + start : nullptr;
+    r.master = d.master ? d.master + start : nullptr;
+    r.count = (uint32_t)count;
+    r.flags = d.flags | (d.dtype == RLX_DTYPE_F32 ? kF32 : 0u);
+    r.pad[0] = r.pad[1] = 0;
+    uint32_t valign = 1;
+    for (uint32_t e = 8; e > 1; e >>= 1) {
+        if (is_aligned(r.p, e * es) && is_aligned(r.g, e * es) && is_aligned(r.m, e * 4) && is_aligned(r.v, e * 4) &&
+            is_aligned(r.master, e * 4)) {
+            valign = e;
+            break;
+        }
+    }
+    r.flags |= valign << kValignShift;
+    return r;
+}
+
+struct UpdateVariant { int tile; };
+
+template <int E, int BLOCK, int K, bool SINGLE>
+void launch_variant(const ChunkRec* recs, const ChunkRec& single, int64_t single_n, int64_t n_elems_or_tiles,
+                    int chunk_log2, const Hyper& h, const NormResult* norm, hipStream_t s) {
+    constexpr int TILE = E * BLOCK;
+    int64_t n_tiles;
+    int tpc_log2 = 0;
+    if constexpr (SINGLE) {
+        n_tiles = (n_elems_or_tiles + TILE - 1) / TILE;
+    } else {
+        tpc_log2 = chunk_log2 - __builtin_ctz(TILE);
+        n_tiles = n_elems_or_tiles << tpc_log2;          // n_chunks * tiles per chunk
+    }
+    for (int64_t first = 0; first < n_tiles; first += kMaxTilesPerLaunch) {
+        int64_t here = n_tiles - first < kMaxTilesPerLaunch ? n_tiles - first : kMaxTilesPerLaunch;
+        here = (here + 8 * K - 1) / (8 * K) * (8 * K);   // whole swizzle groups; the excess exits at once
+        adamw_tile_kernel<E, BLOCK, K, SINGLE><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(
+            recs, single, single_n, first, n_tiles, tpc_log2, h, norm);
+    }
+}
+
 template <bool SINGLE>
-int launch_update(const DevTensor* tensors, const DevChunk* chunks, const DevTensor& single, int64_t n_chunks,
-                  int64_t chunk_elems, const Hyper& h, const NormResult* norm, hipStream_t s) {
-    const dim3 grid((unsigned)pick_grid(n_chunks, g_tuning.update_grid)), block(kBlock);
+int launch_update(const ChunkRec* recs, const ChunkRec& single, int64_t single_n, int64_t n, int chunk_log2,
+                  const Hyper& h, const NormResult* norm, hipStream_t s) {
     switch (g_tuning.update_variant) {
     default:
-    case 0: adamw_update_kernel<4, false, SINGLE><<<grid, block, 0, s>>>(tensors, chunks, single, n_chunks, chunk_elems, h, norm); break;
-    case 1: adamw_update_kernel<4, true, SINGLE><<<grid, block, 0, s>>>(tensors, chunks, single, n_chunks, chunk_elems, h, norm); break;
-    case 2: adamw_update_kernel<2, false, SINGLE><<<grid, block, 0, s>>>(tensors, chunks, single, n_chunks, chunk_elems, h, norm); break;
-    case 3: adamw_update_kernel<2, true, SINGLE><<<grid, block, 0, s>>>(tensors, chunks, single, n_chunks, chunk_elems, h, norm); break;
-    case 4: adamw_update_kernel<1, false, SINGLE><<<grid, block, 0, s>>>(tensors, chunks, single, n_chunks, chunk_elems, h, norm); break;
-    case 5: adamw_update_kernel<1, true, SINGLE><<<grid, block, 0, s>>>(tensors, chunks, single, n_chunks, chunk_elems, h, norm); break;
+    case 0: launch_variant<2, 128, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
+    case 1: launch_variant<2, 128, 2, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
+    case 2: launch_variant<2, 64, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
+    case 3: launch_variant<2, 64, 2, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
+    case 4: launch_variant<4, 64, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
+    case 5: launch_variant<2, 256, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
+    case 6: launch_variant<1, 256, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
+    case 7: launch_variant<4, 128, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
     }
     RLX_HIP(hipGetLastError());
     return RLX_OK;
@@ -604,18 +612,17 @@ int launch_update(const DevTensor* tensors, const DevChunk* chunks, const DevTen
 int flat_update(void* p, const void* g, float* m, float* v, float* master, int64_t n, int dtype,
                 float lr, float beta1, float beta2, float eps, float wd, float bc1, float bc2, void* stream) {
     if (n <= 0) return RLX_OK;                                   // adamw.cu:49,99
+    if (!p || !g || !m || !v) return RLX_ERR_INVALID_ARG;
     rlx_tensor_desc d;
     d.param = p; d.grad = const_cast<void*>(g); d.m = m; d.v = v; d.master = master;
     d.n = n; d.dtype = dtype; d.flags = 0;
-    if (!p || !g || !m || !v) return RLX_ERR_INVALID_ARG;
-    int st = check_hyper(lr, beta1, beta2, eps, wd, bc1, bc2);
+    int st = check_desc(d);
     if (st != RLX_OK) return st;
-    DevTensor t;
-    st = make_dev_tensor(d, t);
+    st = check_hyper(lr, beta1, beta2, eps, wd, bc1, bc2);
     if (st != RLX_OK) return st;
-    const int64_t n_chunks = (n + kDefaultChunk - 1) / kDefaultChunk;
-    return launch_update<true>(nullptr, nullptr, t, n_chunks, kDefaultChunk,
-                               make_hyper(lr, beta1, beta2, eps, wd, bc1, bc2), nullptr, (hipStream_t)stream);
+    const ChunkRec r = make_rec(d, 0, 0);
+    return launch_update<true>(nullptr, r, n, n, 0, make_hyper(lr, beta1, beta2, eps, wd, bc1, bc2), nullptr,
+                               (hipStream_t)stream);
 }
 
 }  // namespace
@@ -623,9 +630,9 @@ int flat_update(void* p, const void* g, float* m, float* v, float* master, int64
 struct rlx_plan {
     uint32_t magic;
     int device;
+    int chunk_log2;
     int64_t n_tensors, n_chunks, n_elems, chunk_elems;
-    DevTensor* d_tensors;
-    DevChunk* d_chunks;
+    ChunkRec* d_recs;
     double* d_partials;
     NormResult* d_norm;
     NormResult* h_norm;      // pinned
@@ -673,9 +680,9 @@ int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream) {
     if (n <= 0) return RLX_OK;
     if (!dst || !src) return RLX_ERR_INVALID_ARG;
     if (!is_aligned(dst, 4) || !is_aligned(src, 2)) return RLX_ERR_MISALIGNED;
-    int64_t grid = (n + kBlock - 1) / kBlock;
+    int64_t grid = (n + 255) / 256;
     if (grid > 65536) grid = 65536;
-    fp16_to_fp32_kernel<<<dim3((unsigned)grid), dim3(kBlock), 0, (hipStream_t)stream>>>(dst, src, n);
+    fp16_to_fp32_kernel<<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(dst, src, n);
     RLX_HIP(hipGetLastError());
     return RLX_OK;
 }
@@ -684,39 +691,43 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
     if (!out) return RLX_ERR_INVALID_ARG;
     *out = nullptr;
     if (!descs || count <= 0 || count > INT32_MAX) return RLX_ERR_INVALID_ARG;
-    if (chunk_elems == 0) chunk_elems = kDefaultChunk;
-    if (chunk_elems < kGroup || chunk_elems % kGroup != 0 || chunk_elems > (1 << 24)) return RLX_ERR_INVALID_ARG;
-
-    std::vector<DevTensor> tensors((size_t)count);
-    int64_t n_chunks = 0, n_elems = 0;
+    int64_t n_elems = 0;
     for (int64_t i = 0; i < count; i++) {
-        int st = make_dev_tensor(descs[i], tensors[(size_t)i]);
+        int st = check_desc(descs[i]);
         if (st != RLX_OK) return st;
-        n_chunks += (descs[i].n + chunk_elems - 1) / chunk_elems;
         n_elems += descs[i].n;
     }
+    // Default: big chunks for big tensors; for a list of many small tensors a smaller chunk
+    // wastes fewer workgroups on the empty part of each tensor's last chunk.
+    if (chunk_elems == 0) chunk_elems = n_elems / count >= 4 * kBigChunk ? kBigChunk : kMinChunk;
+    if (chunk_elems < kMinChunk || chunk_elems > (1 << 24) || (chunk_elems & (chunk_elems - 1)) != 0)
+        return RLX_ERR_INVALID_ARG;
+    int64_t n_chunks = 0;
+    for (int64_t i = 0; i < count; i++) n_chunks += (descs[i].n + chunk_elems - 1) / chunk_elems;
     if (n_chunks > INT32_MAX) return RLX_ERR_TOO_LARGE;
-    std::vector<DevChunk> chunks;
-    chunks.reserve((size_t)n_chunks);
+
+    std::vector<ChunkRec> recs;
+    recs.reserve((size_t)n_chunks);
     for (int64_t i = 0; i < count; i++) {
-        const int64_t k = (descs[i].n + chunk_elems - 1) / chunk_elems;
-        for (int64_t j = 0; j < k; j++) chunks.push_back(DevChunk{(int32_t)i, (int32_t)j});
+        for (int64_t start = 0; start < descs[i].n; start += chunk_elems) {
+            const int64_t left = descs[i].n - start;
+            recs.push_back(make_rec(descs[i], start, left < chunk_elems ? left : chunk_elems));
+        }
     }
 
     rlx_plan* p = new (std::nothrow) rlx_plan();
     if (!p) return RLX_ERR_INVALID_ARG;
     p->magic = kPlanMagic;
+    p->chunk_log2 = __builtin_ctzll((unsigned long long)chunk_elems);
     p->n_tensors = count; p->n_chunks = n_chunks; p->n_elems = n_elems; p->chunk_elems = chunk_elems;
-    p->d_tensors = nullptr; p->d_chunks = nullptr; p->d_partials = nullptr; p->d_norm = nullptr; p->h_norm = nullptr;
+    p->d_recs = nullptr; p->d_partials = nullptr; p->d_norm = nullptr; p->h_norm = nullptr;
 
     hipError_t e = hipGetDevice(&p->device);
-    if (e == hipSuccess) e = hipMalloc((void**)&p->d_tensors, sizeof(DevTensor) * (size_t)count);
-    if (e == hipSuccess) e = hipMalloc((void**)&p->d_chunks, sizeof(DevChunk) * (size_t)n_chunks);
+    if (e == hipSuccess) e = hipMalloc((void**)&p->d_recs, sizeof(ChunkRec) * (size_t)n_chunks);
     if (e == hipSuccess) e = hipMalloc((void**)&p->d_partials, sizeof(double) * (size_t)n_chunks);
     if (e == hipSuccess) e = hipMalloc((void**)&p->d_norm, sizeof(NormResult));
     if (e == hipSuccess) e = hipHostMalloc((void**)&p->h_norm, sizeof(NormResult), hipHostMallocDefault);
-    if (e == hipSuccess) e = hipMemcpy(p->d_tensors, tensors.data(), sizeof(DevTensor) * (size_t)count, hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = hipMemcpy(p->d_chunks, chunks.data(), sizeof(DevChunk) * (size_t)n_chunks, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(p->d_recs, recs.data(), sizeof(ChunkRec) * (size_t)n_chunks, hipMemcpyHostToDevice);
     if (e == hipSuccess) {
         const NormResult init = {0.0, 0.0f, 1.0f};
         *p->h_norm = init;
@@ -735,8 +746,7 @@ int rlx_plan_destroy(rlx_plan* p) {
     if (!p) return RLX_OK;
     if (!plan_ok(p)) return RLX_ERR_INVALID_ARG;
     hipError_t first = hipSuccess, e;
-    if (p->d_tensors && (e = hipFree(p->d_tensors)) != hipSuccess && first == hipSuccess) first = e;
-    if (p->d_chunks && (e = hipFree(p->d_chunks)) != hipSuccess && first == hipSuccess) first = e;
+    if (p->d_recs && (e = hipFree(p->d_recs)) != hipSuccess && first == hipSuccess) first = e;
     if (p->d_partials && (e = hipFree(p->d_partials)) != hipSuccess && first == hipSuccess) first = e;
     if (p->d_norm && (e = hipFree(p->d_norm)) != hipSuccess && first == hipSuccess) first = e;
     if (p->h_norm && (e = hipHostFree(p->h_norm)) != hipSuccess && first == hipSuccess) first = e;
@@ -754,11 +764,14 @@ const double* rlx_plan_partials_device_ptr(const rlx_plan* p) { return plan_ok(p
 int rlx_plan_grad_norm(rlx_plan* p, float max_norm, void* stream) {
     if (!plan_ok(p)) return RLX_ERR_INVALID_ARG;
     hipStream_t s = (hipStream_t)stream;
-    const dim3 grid((unsigned)pick_grid(p->n_chunks, g_tuning.norm_grid)), block(kBlock);
+    int64_t g = g_tuning.norm_grid > 0 ? g_tuning.norm_grid : p->n_chunks;
+    if (g > p->n_chunks) g = p->n_chunks;
+    if (g > kMaxNormGrid) g = kMaxNormGrid;
+    const dim3 grid((unsigned)g), block(kNormBlock);
     if (g_tuning.norm_nt)
-        sumsq_partials_kernel<true><<<grid, block, 0, s>>>(p->d_tensors, p->d_chunks, p->n_chunks, p->chunk_elems, p->d_partials);
+        sumsq_partials_kernel<true><<<grid, block, 0, s>>>(p->d_recs, p->n_chunks, p->d_partials);
     else
-        sumsq_partials_kernel<false><<<grid, block, 0, s>>>(p->d_tensors, p->d_chunks, p->n_chunks, p->chunk_elems, p->d_partials);
+        sumsq_partials_kernel<false><<<grid, block, 0, s>>>(p->d_recs, p->n_chunks, p->d_partials);
     RLX_HIP(hipGetLastError());
     sumsq_final_kernel<<<dim3(1), dim3(kFinalBlock), 0, s>>>(p->d_partials, p->n_chunks, max_norm, p->d_norm);
     RLX_HIP(hipGetLastError());
@@ -778,9 +791,9 @@ int rlx_plan_norm_read(rlx_plan* p, float* norm, float* scale, double* sum_sq, v
 
 int rlx_plan_scale_grads(rlx_plan* p, void* stream) {
     if (!plan_ok(p)) return RLX_ERR_INVALID_ARG;
-    const dim3 grid((unsigned)pick_grid(p->n_chunks, g_tuning.update_grid)), block(kBlock);
-    scale_grads_kernel<false><<<grid, block, 0, (hipStream_t)stream>>>(p->d_tensors, p->d_chunks, p->n_chunks,
-                                                                       p->chunk_elems, p->d_norm);
+    int64_t g = p->n_chunks < kMaxNormGrid ? p->n_chunks : kMaxNormGrid;
+    scale_grads_kernel<<<dim3((unsigned)g), dim3(kNormBlock), 0, (hipStream_t)stream>>>(p->d_recs, p->n_chunks,
+                                                                                      p->d_norm);
     RLX_HIP(hipGetLastError());
     return RLX_OK;
 }
@@ -793,17 +806,18 @@ int rlx_plan_adamw(rlx_plan* p, const rlx_step_params* sp, int clip_mode, void* 
     if (st != RLX_OK) return st;
     const Hyper h = make_hyper(sp->lr, sp->beta1, sp->beta2, sp->eps, sp->weight_decay, sp->bias_correction1,
                                sp->bias_correction2);
-    DevTensor none;
+    ChunkRec none;
     memset(&none, 0, sizeof(none));
-    return launch_update<false>(p->d_tensors, p->d_chunks, none, p->n_chunks, p->chunk_elems, h,
+    return launch_update<false>(p->d_recs, none, 0, p->n_chunks, p->chunk_log2, h,
                                 clip_mode == RLX_CLIP_FUSED ? p->d_norm : nullptr, (hipStream_t)stream);
 }
 
 int rlx_set_tuning(const char* key, int64_t value) {
     if (!key || value < 0) return RLX_ERR_INVALID_ARG;
-    if (!strcmp(key, "update_variant")) { if (value > 5) return RLX_ERR_INVALID_ARG; g_tuning.update_variant = value; }
-    else if (!strcmp(key, "update_grid")) g_tuning.update_grid = value;
-    else if (!strcmp(key, "norm_grid")) g_tuning.norm_grid = value;
+    if (!strcmp(key, "update_variant")) {
+        if (value >= kNumUpdateVariants) return RLX_ERR_INVALID_ARG;
+        g_tuning.update_variant = value;
+    } else if (!strcmp(key, "norm_grid")) g_tuning.norm_grid = value;
     else if (!strcmp(key, "norm_nt")) g_tuning.norm_nt = value ? 1 : 0;
     else return RLX_ERR_INVALID_ARG;
     return RLX_OK;
@@ -812,7 +826,6 @@ int rlx_set_tuning(const char* key, int64_t value) {
 int64_t rlx_get_tuning(const char* key) {
     if (!key) return -1;
     if (!strcmp(key, "update_variant")) return g_tuning.update_variant;
-    if (!strcmp(key, "update_grid")) return g_tuning.update_grid;
     if (!strcmp(key, "norm_grid")) return g_tuning.norm_grid;
     if (!strcmp(key, "norm_nt")) return g_tuning.norm_nt;
     return -1;
@@ -823,13 +836,13 @@ static int fill_common(void* dst, int elem_size, int64_t n, uint64_t seed, int64
     if (n <= 0) return RLX_OK;
     if (!dst || first < 0 || row_len < 0) return RLX_ERR_INVALID_ARG;
     if (!is_aligned(dst, (size_t)elem_size)) return RLX_ERR_MISALIGNED;
-    int64_t grid = (n + kBlock - 1) / kBlock;
+    int64_t grid = (n + kFillBlock - 1) / kFillBlock;
     if (grid > 262144) grid = 262144;
     if (elem_size == 2)
-        fill_kernel<uint16_t><<<dim3((unsigned)grid), dim3(kBlock), 0, (hipStream_t)stream>>>(
+        fill_kernel<uint16_t><<<dim3((unsigned)grid), dim3(kFillBlock), 0, (hipStream_t)stream>>>(
             (uint16_t*)dst, n, seed, first, mean, std, flags, row_len, zero_rows_below);
     else
-        fill_kernel<float><<<dim3((unsigned)grid), dim3(kBlock), 0, (hipStream_t)stream>>>(
+        fill_kernel<float><<<dim3((unsigned)grid), dim3(kFillBlock), 0, (hipStream_t)stream>>>(
             (float*)dst, n, seed, first, mean, std, flags, row_len, zero_rows_below);
     RLX_HIP(hipGetLastError());
     return RLX_OK;
