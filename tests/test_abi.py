@@ -1,0 +1,128 @@
+"""CPU-only checks of the boundary: the shared library loads, exports every symbol that
+include/rlx_adamw.h declares, and rejects bad arguments before touching a device."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "rlx_adamw.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(rlx_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound(B):
+    lib = B.load()
+    names = declared_symbols()
+    assert len(names) >= 20
+    for name in names:
+        assert hasattr(lib, name), name + " is declared in the header but not exported"
+    assert sorted(B.SIGNATURES) == names, "binding and header disagree"
+
+
+def test_header_is_plain_c(tmp_path):
+    """The header compiles as C99 with no HIP or torch headers in reach."""
+    src = tmp_path / "t.c"
+    src.write_text('#include "rlx_adamw.h"\nint main(void){rlx_step_params p; (void)p; return sizeof(rlx_tensor_desc) == 56 ? 0 : 1;}\n')
+    exe = tmp_path / "t"
+    assert os.system("gcc -std=c99 -Wall -Werror -I%s/include -o %s %s" % (ROOT, exe, src)) == 0
+    assert os.system(str(exe)) == 0
+
+
+def test_struct_layouts_match(B):
+    assert C.sizeof(B.TensorDesc) == 56 and C.sizeof(B.StepParams) == 28
+
+
+def test_version_and_status_strings(B):
+    lib = B.load()
+    assert lib.rlx_version() == 100
+    assert lib.rlx_status_string(B.OK) == b"ok"
+    for st in range(1, 7):
+        assert lib.rlx_status_string(st) not in (b"ok", b"unknown status")
+    assert lib.rlx_status_string(99) == b"unknown status"
+
+
+def test_argument_checks_need_no_device(B):
+    hyper = (1e-3, 0.9, 0.999, 1e-8, 0.01, 0.1, 0.001)
+    # n <= 0 is a silent no-op (src/kernels/adamw.cu:49,99)
+    assert B.adamw_fp16(None, None, None, None, None, 0, *hyper) == B.OK
+    assert B.adamw_fp32(None, None, None, None, -1, *hyper) == B.OK
+    assert B.fp16_to_fp32(None, None, 0) == B.OK
+    # null pointers, misalignment, bad hyper-parameters: rejected on the host
+    assert B.adamw_fp16(None, None, None, None, None, 8, *hyper) == B.ERR_INVALID_ARG
+    assert B.adamw_fp16(None, 0x1001, 0x1000, 0x1000, 0x1000, 8, *hyper) == B.ERR_MISALIGNED
+    assert B.adamw_fp32(0x1000, 0x1000, 0x1002, 0x1000, 8, *hyper) == B.ERR_MISALIGNED
+    assert B.adamw_fp16(None, 0x1000, 0x1000, 0x1000, 0x1000, 8, 1e-3, 0.9, 0.999, 1e-8, 0.01, 0.0, 0.001) \
+        == B.ERR_BAD_HYPER
+    assert B.adamw_fp32(0x1000, 0x1000, 0x1000, 0x1000, 8, float("inf"), 0.9, 0.999, 1e-8, 0.0, 0.1, 0.1) \
+        == B.ERR_BAD_HYPER
+    assert B.fp16_to_fp32(0x1000, None, 4) == B.ERR_INVALID_ARG
+
+
+def test_plan_argument_checks(B):
+    lib = B.load()
+    h = C.c_void_p()
+    d = B.TensorDesc(0x1000, 0x2000, 0x3000, 0x4000, None, 100, B.DTYPE_F16, 0)
+    arr = (B.TensorDesc * 1)(d)
+    assert lib.rlx_plan_create(None, 1, 0, C.byref(h)) == B.ERR_INVALID_ARG
+    assert lib.rlx_plan_create(arr, 0, 0, C.byref(h)) == B.ERR_INVALID_ARG
+    assert lib.rlx_plan_create(arr, 1, 3000, C.byref(h)) == B.ERR_INVALID_ARG        # not a power of two
+    assert lib.rlx_plan_create(arr, 1, 1024, C.byref(h)) == B.ERR_INVALID_ARG        # below 2048
+    for bad in (B.TensorDesc(0x1000, 0x2000, 0x3000, 0x4000, None, 0, B.DTYPE_F16, 0),       # n == 0
+                B.TensorDesc(0x1000, None, 0x3000, 0x4000, None, 8, B.DTYPE_F16, 0),          # no gradient
+                B.TensorDesc(None, 0x2000, 0x3000, 0x4000, None, 8, B.DTYPE_F16, 0),          # no parameter
+                B.TensorDesc(0x1000, 0x2000, 0x3000, 0x4000, None, 8, 7, 0),                  # dtype
+                B.TensorDesc(0x1000, 0x2000, 0x3000, 0x4000, None, 8, B.DTYPE_F16, 64),       # flags
+                B.TensorDesc(0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 8, B.DTYPE_F32, 0)):     # master on FP32
+        assert lib.rlx_plan_create((B.TensorDesc * 1)(bad), 1, 0, C.byref(h)) == B.ERR_INVALID_ARG
+    odd = B.TensorDesc(0x1001, 0x2000, 0x3000, 0x4000, None, 8, B.DTYPE_F16, 0)
+    assert lib.rlx_plan_create((B.TensorDesc * 1)(odd), 1, 0, C.byref(h)) == B.ERR_MISALIGNED
+    assert h.value is None
+    assert lib.rlx_plan_destroy(None) == B.OK
+    assert lib.rlx_plan_num_chunks(None) == -1
+    assert lib.rlx_plan_grad_norm(None, 1.0, None) == B.ERR_INVALID_ARG
+    assert lib.rlx_plan_adamw(None, None, 0, None) == B.ERR_INVALID_ARG
+
+
+def test_tuning_keys(B):
+    assert B.get_tuning("update_variant") == 0
+    B.set_tuning("update_variant", 2)
+    assert B.get_tuning("update_variant") == 2
+    B.set_tuning("update_variant", 0)
+    with pytest.raises(B.RlxError):
+        B.set_tuning("update_variant", 99)
+    with pytest.raises(B.RlxError):
+        B.set_tuning("no_such_key", 1)
+    assert B.get_tuning("no_such_key") == -1
+
+
+def test_layouts(L):
+    """Tensor lists of the workloads (shapes of include/model/config.h:6-12; pool order of
+    include/training/optimizer.h:30-32)."""
+    s = L.qwen3_tensor_list(L.QWEN3_0_6B)
+    assert len(s) == 310 and L.total_elements(s) == 596_049_920
+    assert sum(t.n for t in s if t.row_len) == 595_984_384            # the FP16 pool of the reference
+    assert [t.name for t in s[:7]] == ["layers.0." + k for k in
+                                      ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj")]
+    assert s[196].name == "embed_tokens" and s[196].n == 151936 * 1024 and s[-1].name == "final_norm"
+    ref = L.qwen3_tensor_list(L.QWEN3_0_6B, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
+    assert sum(t.n for t in ref if t.dtype == L.DTYPE_F32) == 65_536
+    assert all(t.flags & L.NO_DECAY for t in ref if t.dtype == L.DTYPE_F32 or t.name == "embed_tokens")
+    assert not any(t.flags for t in ref if "proj" in t.name)
+    big = L.qwen3_tensor_list(L.QWEN3_8B)
+    assert len(big) == 399 and L.total_elements(big) == 8_190_427_136 + 308_224
+    r = L.ragged_tensor_list()
+    assert len(r) == 4096 and r == L.ragged_tensor_list()
+    small = sum(1 for t in r if t.n in (128, 1024))
+    assert 0.55 < small / 4096 < 0.65 and min(t.n for t in r) == 128 and max(t.n for t in r) <= 65536
+    assert any(t.n % 8 for t in r)
+
+
+def test_host_bias_correction_matches_oracle(host, O):
+    for beta in (0.9, 0.999, 0.5):
+        for t in (1, 2, 99, 100, 1000):
+            assert host.bias_correction(beta, t) == O.bias_correction(beta, t)

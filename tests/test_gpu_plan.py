@@ -1,0 +1,274 @@
+"""GPU parity of the multi-tensor plan (norm, clip, update) against the CPU oracle, through the
+C ABI.  Sizes here are small enough for the oracle to replay every element."""
+import numpy as np
+import pytest
+
+from util import HYPER, bits, check_state
+
+pytestmark = pytest.mark.gpu
+
+MINI = dict(vocab=1000, hidden=64, inter=192, layers=2, q_heads=4, kv_heads=2, head_dim=16, tied=True)
+
+
+def host_copy(store):
+    """numpy copies of every tensor's p, g, m, v (and master)."""
+    out = []
+    for i in range(len(store.specs)):
+        d = dict(p=bits(store.param(i)), g=bits(store.grad(i)), m=bits(store.state(i, "m")),
+                 v=bits(store.state(i, "v")))
+        if store.master is not None:
+            d["master"] = bits(store.state(i, "master"))
+        out.append(d)
+    return out
+
+
+def oracle_step(O, L, specs, hs, step, hyper, clip_scale=None, master=False):
+    bc1, bc2 = O.bias_correction(hyper["beta1"], step), O.bias_correction(hyper["beta2"], step)
+    for s, h in zip(specs, hs):
+        wd = 0.0 if s.flags & L.NO_DECAY else hyper["wd"]
+        if s.dtype == L.DTYPE_F16:
+            O.adamw_fp16(h.get("master") if master else None, h["p"], h["g"], h["m"], h["v"], hyper["lr"],
+                         hyper["beta1"], hyper["beta2"], hyper["eps"], wd, bc1, bc2, clip_scale=clip_scale)
+        else:
+            O.adamw_fp32(h["p"], h["g"], h["m"], h["v"], hyper["lr"], hyper["beta1"], hyper["beta2"],
+                         hyper["eps"], wd, bc1, bc2, clip_scale=clip_scale)
+
+
+def compare(store, hs, what=""):
+    bad = 0
+    for i, h in enumerate(hs):
+        bad += check_state(bits(store.param(i)), bits(store.state(i, "m")), bits(store.state(i, "v")),
+                           h["p"], h["m"], h["v"], "%s tensor %d" % (what, i))
+        if "master" in h and store.specs[i].dtype == 0:
+            assert np.array_equal(bits(store.state(i, "master")), h["master"])
+    return bad
+
+
+@pytest.mark.parametrize("norm_dtype,ref_groups,master", [(0, False, False), (1, True, False), (1, True, True)])
+def test_model_shaped_list_five_steps(O, L, host, torch_gpu, norm_dtype, ref_groups, master):
+    """A small Qwen3-shaped tensor list (all FP16, or the reference's layout with FP32 norm weights,
+    no decay on embedding and norms, FP32 master copy), five steps with fresh gradients."""
+    torch = torch_gpu
+    specs = L.qwen3_tensor_list(MINI, norm_dtype=norm_dtype, reference_decay_groups=ref_groups)
+    st = host.ParamStore(specs, master=master)
+    st.fill("p", 1, 0.0, 0.02)
+    if master:
+        st.init_master()
+    opt = host.AdamWOptimizer(st, lr=1e-3, weight_decay=0.01, chunk_elems=2048)
+    hyper = dict(HYPER, lr=1e-3)
+    torch.cuda.synchronize()
+    hs = host_copy(st)
+    bad = 0
+    for step in range(1, 6):
+        st.fill("g", 100 + step, 0.0, 1e-4, zero_row_frac=0.9, only=("embed_tokens",))
+        torch.cuda.synchronize()
+        for i, h in enumerate(hs):
+            h["g"] = bits(st.grad(i))
+        opt.step()
+        assert opt.get_step() == step
+        oracle_step(O, L, specs, hs, step, hyper, master=master)
+        torch.cuda.synchronize()
+        bad += compare(st, hs, "step %d" % step)
+    assert bad == 0
+    emb = [i for i, s in enumerate(specs) if s.name == "embed_tokens"][0]
+    g = hs[emb]["g"].reshape(MINI["vocab"], MINI["hidden"])
+    assert 0.8 < (~g.any(axis=1)).mean() < 0.97          # sparse token usage: most rows have zero gradient
+
+
+def test_device_fill_equals_host_fill(O, L, host, torch_gpu):
+    specs = [L.TensorSpec("e", 300 * 64, L.DTYPE_F16, 0, 64), L.TensorSpec("n", 1000, L.DTYPE_F32, 0, 0)]
+    st = host.ParamStore(specs)
+    st.fill("g", 9, 0.0, 1e-2, zero_row_frac=0.5, only=("e",))
+    st.fill("m", 10, 1e-8, 1e-8, flags=1)
+    torch_gpu.cuda.synchronize()
+    thr = int(0.5 * 2 ** 32)
+    assert np.array_equal(bits(st.grad(0)), O.fill_f16(300 * 64, L._hash64(9, 0), 0.0, 1e-2, row_len=64,
+                                                       zero_rows_below=thr))
+    assert np.array_equal(bits(st.grad(1)), O.fill_f32(1000, L._hash64(9, 1), 0.0, 1e-2))
+    assert np.array_equal(bits(st.state(0, "m")), O.fill_f32(300 * 64, L._hash64(10, 0), 1e-8, 1e-8, flags=1))
+
+
+def _norm_oracle(O, hs, chunk):
+    truth = sum(O.sum_sq_half(h["g"]) if h["g"].dtype == np.uint16 else O.sum_sq_float(h["g"]) for h in hs)
+    mirror, parts = O.sumsq_mirror([h["g"] for h in hs], chunk)
+    return truth, mirror, parts
+
+
+@pytest.mark.parametrize("chunk", [2048, 8192])
+def test_grad_norm_and_clip(O, L, host, B, torch_gpu, chunk):
+    """Norm within 1e-5 of the FP64 truth and bit-identical to the restated device order; the same
+    bits on ten runs; fused clip == scale pass + plain step, bit for bit; scaled gradients equal the
+    oracle's scale pass."""
+    torch = torch_gpu
+    specs = L.qwen3_tensor_list(MINI, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
+    extra = torch.empty(777, dtype=torch.float32, device="cuda:0")           # a D_buf-like workspace tail
+    B.fill_f32(extra.data_ptr(), 777, 5, 0.0, 0.3)
+    stores, opts = [], []
+    for _ in range(2):
+        st = host.ParamStore(specs)
+        st.fill("p", 1, 0.0, 0.02)
+        st.fill("g", 2, 0.0, 5e-3)
+        stores.append(st)
+    ex2 = extra.clone()
+    opts = [host.AdamWOptimizer(stores[0], lr=1e-3, chunk_elems=chunk, extra_grad_only=(extra,)),
+            host.AdamWOptimizer(stores[1], lr=1e-3, chunk_elems=chunk, extra_grad_only=(ex2,))]
+    torch.cuda.synchronize()
+    hs = host_copy(stores[0])
+    hs_all = hs + [dict(g=bits(extra))]
+    truth, mirror, parts = _norm_oracle(O, hs_all, chunk)
+    max_norm = 1.0
+    seen = set()
+    for _ in range(10):
+        opts[0].plan.grad_norm(max_norm)
+        seen.add(opts[0].plan.norm_read())
+    assert len(seen) == 1, "norm differs between runs"
+    norm, scale, sum_sq = seen.pop()
+    assert abs(sum_sq - truth) <= 1e-5 * truth
+    assert sum_sq == mirror, "device reduction order differs from its restatement"
+    assert parts.size == opts[0].plan.num_chunks
+    o_scale, o_norm = O.clip_scale(np.float32(truth), max_norm)
+    assert abs(norm - o_norm) <= 1e-5 * o_norm and norm > max_norm
+    assert scale == O.clip_scale(np.float32(sum_sq), max_norm)[0]
+    # unfused: clip_grad_norm_ scales in place, then a plain step
+    got_norm = opts[0].clip_grad_norm_(max_norm)
+    assert got_norm == norm
+    opts[0].step()
+    # fused: gradients untouched, scale applied inside the update
+    assert host.training_step(opts[1], max_norm, fused_clip=True) == norm
+    torch.cuda.synchronize()
+    for i in range(len(specs)):
+        assert np.array_equal(bits(stores[1].grad(i)), hs[i]["g"]), "fused clip must not write gradients"
+    assert np.array_equal(bits(ex2), hs_all[-1]["g"])
+    # oracle: scale pass (both dtypes, workspace tail included), then the update
+    for h in hs_all:
+        if h["g"].dtype == np.uint16:
+            O.scale_half(h["g"], scale)
+        else:
+            O.scale_float(h["g"], scale)
+    for i in range(len(specs)):
+        assert np.array_equal(bits(stores[0].grad(i)), hs[i]["g"]), "scaled gradients, tensor %d" % i
+    assert np.array_equal(bits(extra), hs_all[-1]["g"])
+    oracle_step(O, L, specs, hs, 1, dict(HYPER, lr=1e-3))
+    assert compare(stores[0], hs, "unfused") == 0
+    assert compare(stores[1], hs, "fused") == 0
+
+
+def test_norm_below_threshold_touches_nothing(O, L, host, torch_gpu):
+    torch = torch_gpu
+    specs = [L.TensorSpec("a", 50_000, L.DTYPE_F16, 0, 0), L.TensorSpec("b", 333, L.DTYPE_F32, 0, 0)]
+    st = host.ParamStore(specs)
+    st.fill("g", 3, 0.0, 1e-4)
+    opt = host.AdamWOptimizer(st)
+    torch.cuda.synchronize()
+    before = [bits(st.grad(i)) for i in range(2)]
+    norm = opt.clip_grad_norm_(1.0)
+    opt.plan.scale_grads()                       # even when called anyway: scale is exactly 1
+    torch.cuda.synchronize()
+    _, scale, _ = opt.plan.norm_read()
+    assert 0 < norm < 1.0 and scale == 1.0
+    assert all(np.array_equal(bits(st.grad(i)), before[i]) for i in range(2))
+
+
+def test_non_finite_gradient(O, L, host, torch_gpu):
+    """A NaN gradient gives a NaN norm; the comparison is false, so nothing is scaled
+    (include/training/trainer.h:343) and the update propagates the NaN to that element only."""
+    torch = torch_gpu
+    specs = [L.TensorSpec("a", 5000, L.DTYPE_F16, 0, 0)]
+    st = host.ParamStore(specs)
+    st.fill("p", 1, 0.0, 0.02)
+    st.fill("g", 2, 0.0, 1e-2)
+    st.grad(0)[1234] = float("nan")
+    opt = host.AdamWOptimizer(st, lr=1e-3)
+    norm = host.training_step(opt, 1.0, fused_clip=True)
+    torch.cuda.synchronize()
+    _, scale, _ = opt.plan.norm_read()
+    assert np.isnan(norm) and scale == 1.0
+    p = st.param(0).float().cpu().numpy()
+    assert np.isnan(p[1234]) and np.isfinite(np.delete(p, 1234)).all()
+
+
+def test_ragged_list_equals_flat_tensor(O, L, host, B, torch_gpu):
+    """4,096 tensors of 128..65,536 elements in one launch against one flat tensor with the same
+    values: identical bits, and both equal to the oracle."""
+    torch = torch_gpu
+    specs = L.ragged_tensor_list()
+    total = L.total_elements(specs)
+    st = host.ParamStore(specs)
+    st.fill("p", 1, 1.0, 0.01)
+    st.fill("g", 2, 0.0, 1e-3)
+    torch.cuda.synchronize()
+    hs = host_copy(st)
+    flat_p = torch.cat([st.param(i) for i in range(len(specs))]).contiguous()
+    flat_g = torch.cat([st.grad(i) for i in range(len(specs))]).contiguous()
+    flat_m = torch.zeros(total, dtype=torch.float32, device="cuda:0")
+    flat_v = torch.zeros(total, dtype=torch.float32, device="cuda:0")
+    opt = host.AdamWOptimizer(st, lr=1e-5)
+    assert opt.plan.chunk_elems == 2048                      # small-tensor lists get small chunks
+    opt.step()
+    bc1, bc2 = host.bias_correction(0.9, 1), host.bias_correction(0.999, 1)
+    assert B.adamw_fp16(None, flat_p.data_ptr(), flat_g.data_ptr(), flat_m.data_ptr(), flat_v.data_ptr(), total,
+                        1e-5, 0.9, 0.999, 1e-8, 0.01, bc1, bc2) == B.OK
+    torch.cuda.synchronize()
+    assert torch.equal(torch.cat([st.param(i) for i in range(len(specs))]), flat_p)
+    assert torch.equal(torch.cat([st.state(i, "m") for i in range(len(specs))]), flat_m)
+    assert torch.equal(torch.cat([st.state(i, "v") for i in range(len(specs))]), flat_v)
+    oracle_step(O, L, specs, hs, 1, dict(HYPER))
+    assert compare(st, hs) == 0
+    # padding between tensors is never written
+    used = torch.zeros(st.m.numel(), dtype=torch.bool, device="cuda:0")
+    for i, s in enumerate(specs):
+        used[st.off[i]: st.off[i] + s.n] = True
+    assert not st.m[~used].any().item() and not st.p16[~used[: st.p16.numel()]].any().item()
+
+
+def test_every_tile_shape_and_chunk_size_gives_the_same_bits(L, host, B, torch_gpu):
+    torch = torch_gpu
+    specs = [L.TensorSpec("a", 70_001, L.DTYPE_F16, 0, 0), L.TensorSpec("b", 2049, L.DTYPE_F32, 0, 0),
+             L.TensorSpec("c", 131, L.DTYPE_F16, L.NO_DECAY, 0)]
+    results = []
+    try:
+        for variant, chunk in [(0, 8192), (1, 8192), (2, 2048), (3, 2048), (4, 4096), (5, 65536), (6, 8192),
+                               (7, 2048)]:
+            B.set_tuning("update_variant", variant)
+            st = host.ParamStore(specs)
+            st.fill("p", 1, 0.0, 0.02)
+            st.fill("g", 2, 0.0, 5e-3)
+            opt = host.AdamWOptimizer(st, lr=1e-3, chunk_elems=chunk)
+            host.training_step(opt, 0.05, fused_clip=True)
+            host.training_step(opt, 0.0)
+            torch.cuda.synchronize()
+            results.append([t.clone() for t in (st.p16, st.p32, st.m, st.v)])
+    finally:
+        B.set_tuning("update_variant", 0)
+    for r in results[1:]:
+        assert all(torch.equal(a, b) for a, b in zip(results[0], r))
+
+
+def test_unaligned_tensors_in_a_plan(O, L, host, B, torch_gpu):
+    """Tensors that start at odd element offsets take the element-by-element path."""
+    torch = torch_gpu
+    n = 10_001
+    pool_p = torch.empty(n + 8, dtype=torch.float16, device="cuda:0")
+    pool_g = torch.empty(n + 8, dtype=torch.float16, device="cuda:0")
+    pool_m = torch.zeros(n + 8, dtype=torch.float32, device="cuda:0")
+    pool_v = torch.zeros(n + 8, dtype=torch.float32, device="cuda:0")
+    B.fill_f16(pool_p.data_ptr(), n + 8, 1, 0.0, 0.02)
+    B.fill_f16(pool_g.data_ptr(), n + 8, 2, 0.0, 5e-3)
+    torch.cuda.synchronize()
+    hp, hg = bits(pool_p), bits(pool_g)
+    hm, hv = np.zeros(n + 8, np.float32), np.zeros(n + 8, np.float32)
+    off = 3
+    d = B.TensorDesc(pool_p.data_ptr() + 2 * off, pool_g.data_ptr() + 2 * off, pool_m.data_ptr() + 4 * off,
+                     pool_v.data_ptr() + 4 * off, None, n, B.DTYPE_F16, 0)
+    plan = B.Plan([d], 2048)
+    plan.grad_norm(0.1)
+    norm, scale, sum_sq = plan.norm_read()
+    assert sum_sq == O.sumsq_mirror([hg[off: off + n]], 2048)[0]
+    sp = B.StepParams(1e-3, 0.9, 0.999, 1e-8, 0.01, host.bias_correction(0.9, 1), host.bias_correction(0.999, 1))
+    plan.adamw(sp, B.CLIP_FUSED)
+    torch.cuda.synchronize()
+    sl = slice(off, off + n)
+    O.adamw_fp16(None, hp[sl], hg[sl], hm[sl], hv[sl], 1e-3, 0.9, 0.999, 1e-8, 0.01, sp.bias_correction1,
+                 sp.bias_correction2, clip_scale=scale)
+    assert np.array_equal(bits(pool_p), hp) and np.array_equal(bits(pool_m), hm) and np.array_equal(bits(pool_v), hv)
+    plan.destroy()

@@ -1,0 +1,215 @@
+"""Pins the oracle's AdamW update: against the CPU loops of the reference's own test
+(tests/test_adamw.cu:194-206 and :276-293, restated with numpy FP32 scalars), against
+torch.optim.AdamW (same mathematics, different rounding order), and against closed forms."""
+import numpy as np
+import pytest
+
+B1, B2, EPS = 0.9, 0.999, 1e-8
+
+
+def f32(x):
+    return np.float32(x)
+
+
+def _ref_test_loop_fp16(w0, g, lr, wd):
+    """tests/test_adamw.cu:283-292: step 1, division by the bias corrections."""
+    b1, b2, lr, wd, eps = f32(B1), f32(B2), f32(lr), f32(wd), f32(EPS)
+    bc1, bc2 = f32(1) - b1, f32(1) - b2
+    mi = (f32(1) - b1) * g
+    vi = (f32(1) - b2) * g * g
+    m_hat = mi / bc1
+    v_hat = vi / bc2
+    return w0 * (f32(1) - lr * wd) - lr * m_hat / (np.sqrt(v_hat) + eps)
+
+
+def test_step1_fp16_against_reference_test_loop(O):
+    """Case 2 of the reference's test: q_proj-sized tensor (2,097,152), lr=1e-3, wd=0.01.  Its
+    pass criteria: master max abs err < 1e-6 and FP16 results identical; here the second is
+    'at most 1 ulp, on a vanishing share', because the loop divides where the kernel
+    multiplies by a host reciprocal."""
+    n = 2048 * 1024
+    p = O.fill_f16(n, 21, 0.0, 0.02)
+    g = O.fill_f16(n, 22, 0.0, 1e-3)
+    w0, gf = O.h2f(p), O.h2f(g)
+    want = _ref_test_loop_fp16(w0, gf, 1e-3, 0.01).astype(np.float32)
+    master = w0.copy()
+    m, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    bc1, bc2 = O.bias_correction(B1, 1), O.bias_correction(B2, 1)
+    O.adamw_fp16(master, p, g, m, v, 1e-3, B1, B2, EPS, 0.01, bc1, bc2)
+    assert np.abs(master - want).max() < 1e-6
+    assert np.array_equal(p, O.f2h(master))                      # model weight is f2h(master) exactly
+    mism = p != O.f2h(want)
+    assert mism.mean() < 1e-3
+    a, b = O.h2f(p[mism]), O.h2f(O.f2h(want)[mism])
+    assert (np.abs(a - b) <= np.spacing(np.abs(b).astype(np.float16)).astype(np.float32)).all()
+    # moments as the loop computes them (exact: same two operations)
+    assert np.array_equal(m, ((f32(1) - f32(B1)) * gf).astype(np.float32))
+    assert np.array_equal(v, ((f32(1) - f32(B2)) * gf * gf).astype(np.float32))
+
+
+def test_step1_fp32_against_reference_test_loop(O):
+    """Case 1 of the reference's test: final_norm (1024 FP32 weights), lr=1e-3, no decay; max abs err < 1e-6."""
+    n = 1024
+    w0 = O.fill_f32(n, 31, 1.0, 0.05)
+    g = O.fill_f32(n, 32, 0.0, 1e-2)
+    want = _ref_test_loop_fp16(w0, g, 1e-3, 0.0)
+    w = w0.copy()
+    m, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    O.adamw_fp32(w, g, m, v, 1e-3, B1, B2, EPS, 0.0, O.bias_correction(B1, 1), O.bias_correction(B2, 1))
+    assert np.abs(w - want).max() < 1e-6
+
+
+def test_against_torch_adamw_ten_steps(O):
+    """torch.optim.AdamW (decoupled decay, bias correction) on FP32 CPU tensors: the same
+    mathematics rounded in another order, so agreement to a few FP32 ulps of the state.
+    The betas are exactly representable in FP32: torch forms 1 - beta in double, the reference
+    in FP32 (`1.0f - beta2`, adamw.cu:27), which for beta2 = 0.999 differ by 1.3e-5 relative."""
+    import torch
+    n = 100_000
+    b1, b2 = 0.875, 1.0 - 2.0 ** -8
+    w0 = O.fill_f32(n, 41, 0.0, 0.02)
+    lr, wd = 1e-3, 0.01
+    p = torch.nn.Parameter(torch.from_numpy(w0.copy()))
+    opt = torch.optim.AdamW([p], lr=lr, betas=(b1, b2), eps=EPS, weight_decay=wd, foreach=False, fused=False)
+    w = w0.copy()
+    m, v = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    for step in range(1, 11):
+        g = O.fill_f32(n, 100 + step, 0.0, 1e-3)
+        p.grad = torch.from_numpy(g.copy())
+        opt.step()
+        O.adamw_fp32(w, g, m, v, lr, b1, b2, EPS, wd, O.bias_correction(b1, step), O.bias_correction(b2, step))
+        st = opt.state[p]
+        tm, tv = st["exp_avg"].numpy(), st["exp_avg_sq"].numpy()
+        assert np.abs(m - tm).max() <= 4e-7 * np.abs(tm).max()
+        assert (np.abs(v - tv) <= 1e-6 * np.abs(tv) + 1e-30).all()
+        assert np.abs(w - p.detach().numpy()).max() <= 2e-6 * lr * step + 1e-8
+    # a dropped bias correction, a wrong sign or coupled decay would be orders of magnitude outside
+    assert np.abs(w - w0).max() > 5 * lr
+
+
+def test_closed_forms(O):
+    n = 4096
+    w0 = O.fill_f32(n, 51, 0.5, 0.1)
+    zeros = np.zeros(n, np.float32)
+    # zero gradient, zero moments, no decay: nothing moves, bit for bit (frozen embedding)
+    w, m, v = w0.copy(), zeros.copy(), zeros.copy()
+    for t in range(1, 4):
+        O.adamw_fp32(w, zeros, m, v, 1e-3, B1, B2, EPS, 0.0, O.bias_correction(B1, t), O.bias_correction(B2, t))
+    assert np.array_equal(w, w0) and not m.any() and not v.any()
+    # zero gradient with decay: w0 * (1 - lr*wd)^t, rounded once per step
+    w = w0.copy()
+    want = w0.copy()
+    factor = f32(1) - f32(1e-2) * f32(0.1)
+    for t in range(1, 6):
+        O.adamw_fp32(w, zeros, m, v, 1e-2, B1, B2, EPS, 0.1, O.bias_correction(B1, t), O.bias_correction(B2, t))
+        want = (want * factor).astype(np.float32)
+    assert np.array_equal(w, want)
+    assert np.allclose(w, w0 * (1 - 1e-2 * 0.1) ** 5, rtol=1e-6)
+    # first step with |g| >> eps and no decay is a sign step of size lr
+    g = O.fill_f32(n, 52, 0.0, 1.0)
+    g[np.abs(g) < 1e-3] = 1e-3
+    w, m, v = w0.copy(), zeros.copy(), zeros.copy()
+    O.adamw_fp32(w, g, m, v, 1e-3, B1, B2, EPS, 0.0, O.bias_correction(B1, 1), O.bias_correction(B2, 1))
+    assert np.abs((w - w0) + 1e-3 * np.sign(g)).max() < 1e-3 * 1e-4 + 1e-7
+
+
+def test_moments_do_not_depend_on_lr_wd_eps(O):
+    n = 10_000
+    g = O.fill_f16(n, 61, 0.0, 1e-3)
+    outs = []
+    for lr, wd, eps in ((1e-5, 0.01, 1e-8), (3e-2, 0.3, 1e-3)):
+        p = O.fill_f16(n, 62, 0.0, 0.02)
+        m, v = O.fill_f32(n, 63, 0.0, 1e-4), O.fill_f32(n, 64, 1e-8, 1e-8, flags=O.FILL_ABS)
+        O.adamw_fp16(None, p, g, m, v, lr, B1, B2, eps, wd, 0.5, 0.25)
+        outs.append((m, v))
+    assert np.array_equal(outs[0][0], outs[1][0]) and np.array_equal(outs[0][1], outs[1][1])
+
+
+def test_elementwise_independence(O):
+    """Any slicing or permutation of the tensor gives the same value per element."""
+    n = 50_000
+    rng = np.random.default_rng(3)
+    perm = rng.permutation(n)
+    p, g = O.fill_f16(n, 71, 0.0, 0.02), O.fill_f16(n, 72, 0.0, 1e-3)
+    m, v = O.fill_f32(n, 73, 0.0, 1e-4), O.fill_f32(n, 74, 1e-8, 1e-8, flags=O.FILL_ABS)
+    args = (1e-4, B1, B2, EPS, 0.01, O.bias_correction(B1, 7), O.bias_correction(B2, 7))
+    a = [x.copy() for x in (p, g, m, v)]
+    O.adamw_fp16(None, a[0], a[1], a[2], a[3], *args)
+    b = [np.ascontiguousarray(x[perm]) for x in (p, g, m, v)]
+    O.adamw_fp16(None, b[0], b[1], b[2], b[3], *args)
+    for x, y in zip(a, b):
+        assert np.array_equal(x[perm], y)
+    c = [x.copy() for x in (p, g, m, v)]
+    for lo, hi in ((0, 1), (1, 4097), (4097, n)):
+        O.adamw_fp16(None, c[0][lo:hi], c[1][lo:hi], c[2][lo:hi], c[3][lo:hi], *args)
+    for x, y in zip(a, c):
+        assert np.array_equal(x, y)
+
+
+def test_master_mode_and_masterless_mode(O):
+    """With a master copy the FP16 weight is never read (Q: adamw.cu:35-39); without one the FP16
+    weight is the source of truth.  The two agree for one step when master == h2f(weight)."""
+    n = 8192
+    p0, g = O.fill_f16(n, 81, 0.0, 0.02), O.fill_f16(n, 82, 0.0, 1e-3)
+    args = (1e-3, B1, B2, EPS, 0.01, O.bias_correction(B1, 1), O.bias_correction(B2, 1))
+    pa, ma, va = p0.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    O.adamw_fp16(None, pa, g, ma, va, *args)
+    garbage = np.full(n, 0x3C00, np.uint16)
+    master, mb, vb = O.h2f(p0), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    O.adamw_fp16(master, garbage, g, mb, vb, *args)
+    assert np.array_equal(garbage, pa) and np.array_equal(ma, mb) and np.array_equal(va, vb)
+    assert np.array_equal(O.f2h(master), garbage)
+
+
+def test_bias_correction(O):
+    # step 1 gives 1 - beta exactly, as the reference's test assumes (tests/test_adamw.cu:196-197)
+    assert O.bias_correction(B1, 1) == float(f32(1) - f32(B1))
+    assert O.bias_correction(B2, 1) == float(f32(1) - f32(B2))
+    for t in (2, 10, 100, 1000, 100000):
+        for b in (B1, B2):
+            want = 1.0 - float(f32(b)) ** t        # beta is an FP32 value on the reference's host
+            assert abs(O.bias_correction(b, t) - want) <= 2e-7 * max(want, 1e-3) + 1e-7
+    assert O.bias_correction(B1, 100000) == 1.0
+
+
+def test_optimizer_step_groups(O):
+    """optimizer.h:119-147: step counter first; decay on projections only; embedding and FP32 norm
+    pools get weight_decay 0 whatever the configured value."""
+    n16, proj_n, n32 = 3000, 2000, 300
+    pool16 = O.fill_f16(n16, 91, 0.0, 0.5)
+    master = O.h2f(pool16)
+    g16 = np.zeros(n16, np.uint16)
+    pool32, g32 = O.fill_f32(n32, 92, 1.0, 0.1), np.zeros(n32, np.float32)
+    m16, v16 = np.zeros(n16, np.float32), np.zeros(n16, np.float32)
+    m32, v32 = np.zeros(n32, np.float32), np.zeros(n32, np.float32)
+    before16, before32 = master.copy(), pool32.copy()
+    step = O.optimizer_step(master, pool16, g16, m16, v16, proj_n, pool32, g32, m32, v32,
+                            1e-2, B1, B2, EPS, 0.1, 0)
+    assert step == 1
+    factor = f32(1) - f32(1e-2) * f32(0.1)
+    assert np.array_equal(master[:proj_n], (before16[:proj_n] * factor).astype(np.float32))
+    assert np.array_equal(master[proj_n:], before16[proj_n:])
+    assert np.array_equal(pool32, before32)
+    assert O.optimizer_step(master, pool16, g16, m16, v16, proj_n, pool32, g32, m32, v32,
+                            1e-2, B1, B2, EPS, 0.1, step) == 2
+
+
+@pytest.mark.parametrize("n", [0, -3])
+def test_non_positive_n_is_a_no_op(O, n):
+    # adamw.cu:49,99: returns before touching anything, even null pointers
+    O.lib.orc_adamw_fp16(None, None, None, None, None, n, 1e-3, B1, B2, EPS, 0.0, 0.1, 0.001)
+    O.lib.orc_adamw_fp32(None, None, None, None, n, 1e-3, B1, B2, EPS, 0.0, 0.1, 0.001)
+
+
+def test_threaded_step_matches_single_thread(O):
+    n = 100_003
+    p, g = O.fill_f16(n, 95, 0.0, 0.02), O.fill_f16(n, 96, 0.0, 5e-3)
+    args = (1e-3, B1, B2, EPS, 0.01, O.bias_correction(B1, 3), O.bias_correction(B2, 3))
+    pa, ma, va = p.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    ga = g.copy()
+    norm, scale = O.clip_grad_norm(ga, None, 1.0)
+    O.adamw_fp16(None, pa, ga, ma, va, *args)
+    pb, mb, vb = p.copy(), np.zeros(n, np.float32), np.zeros(n, np.float32)
+    norm_b = O.step_fp16_threaded(None, pb, g, mb, vb, *args, 1.0, 5)
+    assert abs(norm_b - norm) <= 1e-6 * norm and norm > 1.0
+    assert np.array_equal(pa, pb) and np.array_equal(ma, mb) and np.array_equal(va, vb)
