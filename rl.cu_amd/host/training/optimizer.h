@@ -1,0 +1,200 @@
+// AdamWOptimizer for C++ callers: the reference's class (include/training/optimizer.h:59-274)
+// with the same public members and methods, built from flat pools instead of a Qwen3Model*.
+//
+// Like the reference it owns the FP32 state as flat buffers co-indexed with the weight pools:
+// [master | m | v] for the FP16 pool and [m | v] for the FP32 pool, zero-filled, master
+// initialised from the FP16 weights.  step() increments the step counter, forms the bias
+// corrections with powf on the host and updates every parameter; where the reference issues
+// three launches (projections with decay, embedding and norm weights without), this issues
+// one multi-tensor launch with the same three groups.
+#pragma once
+#include <cassert>
+#include <cmath>
+#include <cstring>
+
+#include "../kernels/adamw.h"
+
+#ifndef HIP_CHECK
+#define HIP_CHECK(x)                                                                                        \
+    do {                                                                                                    \
+        hipError_t err_ = (x);                                                                              \
+        if (err_ != hipSuccess) {                                                                           \
+            fprintf(stderr, "HIP error %s at %s:%d\n", hipGetErrorString(err_), __FILE__, __LINE__);        \
+            exit(1);                                                                                        \
+        }                                                                                                   \
+    } while (0)
+#endif
+
+// The weight pools of the model (Qwen3Weights::fp16_pool / fp32_pool, include/model/weights.h:43-61).
+// The FP16 pool is [projections of all layers | embedding]; proj_elems is the size of the first part.
+struct ParamPools {
+    half* fp16_pool = nullptr;
+    size_t fp16_pool_elems = 0;
+    size_t proj_elems = 0;
+    float* fp32_pool = nullptr;
+    size_t fp32_pool_elems = 0;
+};
+
+// The gradient pools (Qwen3Gradients, include/model/qwen3.h:190-218).  float_pool may be longer
+// than the FP32 weight pool: the reference keeps an attention-backward workspace behind the norm
+// gradients, and its clip includes that tail in the norm and scales it.
+struct GradPools {
+    half* half_pool = nullptr;
+    float* float_pool = nullptr;
+    size_t half_pool_bytes = 0;
+    size_t float_pool_bytes = 0;
+};
+
+class AdamWOptimizer {
+public:
+    // Hyper-parameters (public, as in the reference)
+    float lr;
+    float beta1;
+    float beta2;
+    float eps;
+    float weight_decay;
+
+    AdamWOptimizer() : lr(1e-5f), beta1(0.9f), beta2(0.999f), eps(1e-8f), weight_decay(0.01f) {}
+
+    // use_master = true keeps the reference's FP32 master copy (28 bytes per parameter and step);
+    // false reads the FP16 weight as the source of truth (22 bytes).
+    explicit AdamWOptimizer(const ParamPools& pools, float lr = 1e-4f, float beta1 = 0.9f, float beta2 = 0.999f,
+                            float eps = 1e-8f, float weight_decay = 0.01f, bool use_master = true)
+        : lr(lr), beta1(beta1), beta2(beta2), eps(eps), weight_decay(weight_decay) {
+        init(pools, use_master);
+    }
+
+    ~AdamWOptimizer() { free(); }
+
+    AdamWOptimizer(const AdamWOptimizer&) = delete;
+    AdamWOptimizer& operator=(const AdamWOptimizer&) = delete;
+    AdamWOptimizer(AdamWOptimizer&& o) noexcept { move_from(o); }
+    AdamWOptimizer& operator=(AdamWOptimizer&& o) noexcept {
+        if (this != &o) { free(); move_from(o); }
+        return *this;
+    }
+
+    void set_lr(float new_lr) { lr = new_lr; }
+    int get_step() const { return step_; }
+
+    float* fp16_master() { return fp16_master_; }
+    float* fp16_m() { return fp16_m_; }
+    float* fp16_v() { return fp16_v_; }
+    float* fp32_m() { return fp32_m_; }
+    float* fp32_v() { return fp32_v_; }
+    size_t num_fp16_params() const { return n16_; }
+    size_t num_fp32_params() const { return n32_; }
+
+    // One optimizer step.  fused_clip: apply the clip scale that the last norm pass of
+    // plan_for(grads) left on the device, inside the update (gradients are not written).
+    void step(GradPools* grads, hipStream_t stream = 0, bool fused_clip = false) {
+        step_++;
+        rlx_step_params sp;
+        sp.lr = lr; sp.beta1 = beta1; sp.beta2 = beta2; sp.eps = eps; sp.weight_decay = weight_decay;
+        sp.bias_correction1 = 1.0f - powf(beta1, (float)step_);
+        sp.bias_correction2 = 1.0f - powf(beta2, (float)step_);
+        RLX_CHECK(rlx_plan_adamw(plan_for(grads), &sp, fused_clip ? RLX_CLIP_FUSED : RLX_CLIP_NONE, (void*)stream));
+    }
+
+    // The multi-tensor plan over {projections, embedding, norm weights, workspace tail} for these
+    // gradient pools; built on first use and rebuilt if the pools move.
+    rlx_plan* plan_for(GradPools* grads) {
+        if (plan_ && grads->half_pool == plan_half_ && grads->float_pool == plan_float_ &&
+            grads->float_pool_bytes == plan_float_bytes_)
+            return plan_;
+        if (plan_) { RLX_CHECK(rlx_plan_destroy(plan_)); plan_ = nullptr; }
+        assert(grads->half_pool_bytes / sizeof(half) == n16_);
+        assert(grads->float_pool_bytes / sizeof(float) >= n32_);
+        rlx_tensor_desc d[4];
+        int k = 0;
+        const size_t embed_n = n16_ - proj_n_;
+        if (proj_n_) {
+            d[k++] = {pools_.fp16_pool, grads->half_pool, fp16_m_, fp16_v_, fp16_master_, (int64_t)proj_n_,
+                      RLX_DTYPE_F16, 0};
+        }
+        if (embed_n) {   // no decay on the embedding (optimizer.h:131-140)
+            d[k++] = {pools_.fp16_pool + proj_n_, grads->half_pool + proj_n_, fp16_m_ + proj_n_, fp16_v_ + proj_n_,
+                      fp16_master_ ? fp16_master_ + proj_n_ : nullptr, (int64_t)embed_n, RLX_DTYPE_F16,
+                      RLX_TENSOR_NO_DECAY};
+        }
+        if (n32_) {      // no decay on the norm weights (optimizer.h:142-146)
+            d[k++] = {pools_.fp32_pool, grads->float_pool, fp32_m_, fp32_v_, nullptr, (int64_t)n32_, RLX_DTYPE_F32,
+                      RLX_TENSOR_NO_DECAY};
+        }
+        const size_t tail = grads->float_pool_bytes / sizeof(float) - n32_;
+        if (tail) {
+            d[k++] = {nullptr, grads->float_pool + n32_, nullptr, nullptr, nullptr, (int64_t)tail, RLX_DTYPE_F32,
+                      RLX_TENSOR_GRAD_ONLY};
+        }
+        RLX_CHECK(rlx_plan_create(d, k, 0, &plan_));
+        plan_half_ = grads->half_pool; plan_float_ = grads->float_pool; plan_float_bytes_ = grads->float_pool_bytes;
+        return plan_;
+    }
+
+private:
+    ParamPools pools_;
+    int step_ = 0;
+    float* fp16_master_ = nullptr;
+    float* fp16_m_ = nullptr;
+    float* fp16_v_ = nullptr;
+    float* fp32_m_ = nullptr;
+    float* fp32_v_ = nullptr;
+    float* fp16_state_ = nullptr;   // single allocation: [master | m | v] or [m | v]
+    float* fp32_state_ = nullptr;   // single allocation: [m | v]
+    size_t n16_ = 0, n32_ = 0, proj_n_ = 0;
+    rlx_plan* plan_ = nullptr;
+    half* plan_half_ = nullptr;
+    float* plan_float_ = nullptr;
+    size_t plan_float_bytes_ = 0;
+
+    void init(const ParamPools& pools, bool use_master) {
+        pools_ = pools;
+        n16_ = pools.fp16_pool_elems;
+        n32_ = pools.fp32_pool_elems;
+        proj_n_ = pools.proj_elems;
+        assert(proj_n_ <= n16_);
+        const size_t parts = use_master ? 3 : 2;
+        if (n16_) {
+            HIP_CHECK(hipMalloc((void**)&fp16_state_, n16_ * parts * sizeof(float)));
+            HIP_CHECK(hipMemset(fp16_state_, 0, n16_ * parts * sizeof(float)));
+        }
+        if (n32_) {
+            HIP_CHECK(hipMalloc((void**)&fp32_state_, n32_ * 2 * sizeof(float)));
+            HIP_CHECK(hipMemset(fp32_state_, 0, n32_ * 2 * sizeof(float)));
+        }
+        float* q = fp16_state_;
+        if (use_master) { fp16_master_ = q; q += n16_; }
+        fp16_m_ = q;
+        fp16_v_ = q + n16_;
+        fp32_m_ = fp32_state_;
+        fp32_v_ = fp32_state_ + n32_;
+        if (use_master && n16_) {
+            RLX_CHECK(rlx_fp16_to_fp32(fp16_master_, reinterpret_cast<const uint16_t*>(pools.fp16_pool),
+                                       (int64_t)n16_, nullptr));
+        }
+        HIP_CHECK(hipDeviceSynchronize());
+        printf("[AdamW] Flat buffers: fp16=%zu params (%.1f MB state)  fp32=%zu params (%.2f MB state)  "
+               "(lr=%.1e wd=%.2f)\n",
+               n16_, n16_ * parts * sizeof(float) / (1024.0 * 1024.0), n32_,
+               n32_ * 2 * sizeof(float) / (1024.0 * 1024.0), lr, weight_decay);
+    }
+
+    void free() {
+        if (plan_) { rlx_plan_destroy(plan_); plan_ = nullptr; }
+        if (fp16_state_) { (void)hipFree(fp16_state_); fp16_state_ = nullptr; }
+        if (fp32_state_) { (void)hipFree(fp32_state_); fp32_state_ = nullptr; }
+        fp16_master_ = fp16_m_ = fp16_v_ = fp32_m_ = fp32_v_ = nullptr;
+    }
+
+    void move_from(AdamWOptimizer& o) {
+        lr = o.lr; beta1 = o.beta1; beta2 = o.beta2; eps = o.eps; weight_decay = o.weight_decay;
+        pools_ = o.pools_; step_ = o.step_;
+        fp16_master_ = o.fp16_master_; fp16_m_ = o.fp16_m_; fp16_v_ = o.fp16_v_;
+        fp32_m_ = o.fp32_m_; fp32_v_ = o.fp32_v_;
+        fp16_state_ = o.fp16_state_; fp32_state_ = o.fp32_state_;
+        n16_ = o.n16_; n32_ = o.n32_; proj_n_ = o.proj_n_;
+        plan_ = o.plan_; plan_half_ = o.plan_half_; plan_float_ = o.plan_float_; plan_float_bytes_ = o.plan_float_bytes_;
+        o.plan_ = nullptr; o.fp16_state_ = nullptr; o.fp32_state_ = nullptr;
+        o.fp16_master_ = o.fp16_m_ = o.fp16_v_ = o.fp32_m_ = o.fp32_v_ = nullptr;
+    }
+};

@@ -1,0 +1,253 @@
+// test_adamw_host.cpp
+//
+// C++ host-side test of the optimizer path on a GPU, shaped like the reference's
+// tests/test_adamw.cu (standalone executable, PASS/FAIL lines, exit code = failures), but on
+// seeded synthetic weights and gradients instead of a loaded model:
+//   1. FP32 AdamW vs an inline CPU loop (step 1, no decay)            max err < 1e-6
+//   2. FP16 AdamW vs an inline CPU loop and vs the C oracle           master err < 1e-6; oracle: identical bits
+//   3. moments finite and non-zero after a step
+//   4. get_step() counts 0 -> 3
+//   5. clip_grad_norm_ returns the pre-clip norm; clipped gradients have norm <= max; fused == unfused
+//   6. operator API (launch_adamw_fp16 / launch_adamw_fp32) on raw pointers
+// The oracle (liborc_adamw.so) is used as the checker only.
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <vector>
+
+#include "training/trainer.h"
+
+extern "C" {
+float orc_h2f(uint16_t h);
+uint16_t orc_f2h(float f);
+void orc_adamw_fp16(float*, uint16_t*, const uint16_t*, float*, float*, int64_t, float, float, float, float, float,
+                    float, float);
+void orc_adamw_fp16_clip(float*, uint16_t*, const uint16_t*, float*, float*, int64_t, float, float, float, float,
+                         float, float, float, float, int);
+void orc_adamw_fp32(float*, const float*, float*, float*, int64_t, float, float, float, float, float, float, float);
+float orc_clip_grad_norm(uint16_t*, int64_t, float*, int64_t, float, float*);
+double orc_sum_sq_half(const uint16_t*, int64_t);
+double orc_sum_sq_float(const float*, int64_t);
+}
+
+static int g_fails = 0;
+#define PASS(name) printf("[PASS] %s\n", (name))
+#define FAIL(name, ...) do { printf("[FAIL] %s: ", (name)); printf(__VA_ARGS__); printf("\n"); g_fails++; } while (0)
+
+// A small model-shaped pool set: projections, embedding, norm weights, and a workspace tail
+// behind the norm gradients.
+struct Fixture {
+    size_t proj_n = 3 * 8192 + 1024, embed_n = 500 * 64, n32 = 2304 + 64, tail = 777;
+    size_t n16 = proj_n + embed_n;
+    half *w16 = nullptr, *g16 = nullptr;
+    float *w32 = nullptr, *g32 = nullptr;
+    ParamPools pools;
+    GradPools grads;
+    std::vector<uint16_t> h_w16, h_g16;
+    std::vector<float> h_w32, h_g32;
+
+    explicit Fixture(float grad_std) {
+        HIP_CHECK(hipMalloc((void**)&w16, n16 * 2));
+        HIP_CHECK(hipMalloc((void**)&g16, n16 * 2));
+        HIP_CHECK(hipMalloc((void**)&w32, n32 * 4));
+        HIP_CHECK(hipMalloc((void**)&g32, (n32 + tail) * 4));
+        RLX_CHECK(rlx_fill_f16((uint16_t*)w16, n16, 1, 0, 0.0f, 0.02f, 0, 0, 0, nullptr));
+        RLX_CHECK(rlx_fill_f16((uint16_t*)g16, n16, 2, 0, 0.0f, grad_std, 0, 0, 0, nullptr));
+        RLX_CHECK(rlx_fill_f32(w32, n32, 3, 0, 1.0f, 0.05f, 0, 0, 0, nullptr));
+        RLX_CHECK(rlx_fill_f32(g32, n32 + tail, 4, 0, 0.0f, grad_std, 0, 0, 0, nullptr));
+        HIP_CHECK(hipDeviceSynchronize());
+        pools.fp16_pool = w16; pools.fp16_pool_elems = n16; pools.proj_elems = proj_n;
+        pools.fp32_pool = w32; pools.fp32_pool_elems = n32;
+        grads.half_pool = g16; grads.half_pool_bytes = n16 * 2;
+        grads.float_pool = g32; grads.float_pool_bytes = (n32 + tail) * 4;
+        h_w16.resize(n16); h_g16.resize(n16); h_w32.resize(n32); h_g32.resize(n32 + tail);
+        download();
+    }
+    void download() {
+        HIP_CHECK(hipMemcpy(h_w16.data(), w16, n16 * 2, hipMemcpyDeviceToHost));
+        HIP_CHECK(hipMemcpy(h_g16.data(), g16, n16 * 2, hipMemcpyDeviceToHost));
+        HIP_CHECK(hipMemcpy(h_w32.data(), w32, n32 * 4, hipMemcpyDeviceToHost));
+        HIP_CHECK(hipMemcpy(h_g32.data(), g32, (n32 + tail) * 4, hipMemcpyDeviceToHost));
+    }
+    ~Fixture() { (void)hipFree(w16); (void)hipFree(g16); (void)hipFree(w32); (void)hipFree(g32); }
+};
+
+template <typename T> static std::vector<T> d2h(const T* d, size_t n) {
+    std::vector<T> h(n);
+    HIP_CHECK(hipMemcpy(h.data(), d, n * sizeof(T), hipMemcpyDeviceToHost));
+    return h;
+}
+
+// 1. FP32 path vs the CPU loop of the reference's test (step 1, division by the bias corrections)
+static void test_cpu_reference_fp32() {
+    const char* name = "CPU reference: FP32 AdamW (norm weights)";
+    Fixture f(1e-2f);
+    AdamWOptimizer opt(f.pools, /*lr=*/1e-3f);
+    float bc1 = 1.0f - opt.beta1, bc2 = 1.0f - opt.beta2;
+    std::vector<float> cpu_w(f.n32);
+    for (size_t i = 0; i < f.n32; i++) {
+        float g = f.h_g32[i];
+        float mi = (1.0f - opt.beta1) * g, vi = (1.0f - opt.beta2) * g * g;
+        float m_hat = mi / bc1, v_hat = vi / bc2;
+        cpu_w[i] = f.h_w32[i] - opt.lr * m_hat / (sqrtf(v_hat) + opt.eps);
+    }
+    opt.step(&f.grads);
+    HIP_CHECK(hipDeviceSynchronize());
+    auto gpu_w = d2h(f.w32, f.n32);
+    float max_err = 0.0f;
+    for (size_t i = 0; i < f.n32; i++) max_err = fmaxf(max_err, fabsf(gpu_w[i] - cpu_w[i]));
+    printf("  max_err(GPU vs CPU) = %.8e\n", max_err);
+    if (max_err < 1e-6f) PASS(name); else FAIL(name, "max_err=%.8e", max_err);
+}
+
+// 2. FP16 path (projections: decay 0.01) vs the inline loop and vs the oracle
+static void test_cpu_reference_fp16() {
+    const char* name = "CPU reference: FP16 AdamW (projections)";
+    Fixture f(1e-3f);
+    AdamWOptimizer opt(f.pools, 1e-3f, 0.9f, 0.999f, 1e-8f, 0.01f);
+    const size_t n = f.proj_n;
+    float bc1 = 1.0f - opt.beta1, bc2 = 1.0f - opt.beta2;
+    std::vector<float> cpu_master(n);
+    for (size_t i = 0; i < n; i++) {
+        float g = orc_h2f(f.h_g16[i]);
+        float mi = (1.0f - opt.beta1) * g, vi = (1.0f - opt.beta2) * g * g;
+        float m_hat = mi / bc1, v_hat = vi / bc2;
+        cpu_master[i] = orc_h2f(f.h_w16[i]) * (1.0f - opt.lr * opt.weight_decay) - opt.lr * m_hat / (sqrtf(v_hat) + opt.eps);
+    }
+    // oracle: whole FP16 pool, embedding without decay (optimizer.h:131-140)
+    std::vector<float> o_master(f.n16), o_m(f.n16, 0.0f), o_v(f.n16, 0.0f);
+    for (size_t i = 0; i < f.n16; i++) o_master[i] = orc_h2f(f.h_w16[i]);
+    std::vector<uint16_t> o_w = f.h_w16;
+    orc_adamw_fp16(o_master.data(), o_w.data(), f.h_g16.data(), o_m.data(), o_v.data(), n, opt.lr, opt.beta1,
+                   opt.beta2, opt.eps, opt.weight_decay, bc1, bc2);
+    orc_adamw_fp16(o_master.data() + n, o_w.data() + n, f.h_g16.data() + n, o_m.data() + n, o_v.data() + n,
+                   f.n16 - n, opt.lr, opt.beta1, opt.beta2, opt.eps, 0.0f, bc1, bc2);
+    opt.step(&f.grads);
+    HIP_CHECK(hipDeviceSynchronize());
+    auto gpu_w = d2h((const uint16_t*)f.w16, f.n16);
+    auto gpu_master = d2h(opt.fp16_master(), f.n16);
+    auto gpu_m = d2h(opt.fp16_m(), f.n16);
+    auto gpu_v = d2h(opt.fp16_v(), f.n16);
+    float max_err_master = 0.0f;
+    for (size_t i = 0; i < n; i++) max_err_master = fmaxf(max_err_master, fabsf(gpu_master[i] - cpu_master[i]));
+    size_t vs_oracle = 0, not_f2h = 0;
+    for (size_t i = 0; i < f.n16; i++) {
+        if (gpu_w[i] != o_w[i] || memcmp(&gpu_master[i], &o_master[i], 4) || memcmp(&gpu_m[i], &o_m[i], 4) ||
+            memcmp(&gpu_v[i], &o_v[i], 4))
+            vs_oracle++;
+        if (gpu_w[i] != orc_f2h(gpu_master[i])) not_f2h++;
+    }
+    printf("  master max_err=%.8e  mismatches vs oracle=%zu/%zu  model!=f2h(master): %zu\n", max_err_master,
+           vs_oracle, f.n16, not_f2h);
+    if (max_err_master < 1e-6f && vs_oracle == 0 && not_f2h == 0) PASS(name);
+    else FAIL(name, "master_err=%.8e oracle_mismatch=%zu", max_err_master, vs_oracle);
+}
+
+// 3. moments are finite and non-zero after a step
+static void test_moments_nonzero() {
+    const char* name = "Moments non-zero after step";
+    Fixture f(1e-3f);
+    AdamWOptimizer opt(f.pools, 1e-4f);
+    opt.step(&f.grads);
+    HIP_CHECK(hipDeviceSynchronize());
+    auto m = d2h(opt.fp16_m(), f.n16);
+    auto v = d2h(opt.fp32_v(), f.n32);
+    size_t nz_m = 0, nz_v = 0, bad = 0;
+    for (float x : m) { nz_m += x != 0.0f; bad += !std::isfinite(x); }
+    for (float x : v) { nz_v += x != 0.0f; bad += !std::isfinite(x); }
+    if (bad == 0 && nz_m > f.n16 / 2 && nz_v > f.n32 / 2) PASS(name); else FAIL(name, "nz_m=%zu nz_v=%zu bad=%zu", nz_m, nz_v, bad);
+}
+
+// 4. step counter
+static void test_step_counter() {
+    const char* name = "get_step() counts steps";
+    Fixture f(1e-3f);
+    AdamWOptimizer opt(f.pools, 1e-4f);
+    bool ok = opt.get_step() == 0;
+    for (int i = 0; i < 3; i++) opt.step(&f.grads);
+    HIP_CHECK(hipDeviceSynchronize());
+    ok = ok && opt.get_step() == 3;
+    AdamWOptimizer moved(std::move(opt));
+    ok = ok && moved.get_step() == 3 && opt.fp16_m() == nullptr;
+    moved.set_lr(5e-5f);
+    ok = ok && moved.lr == 5e-5f;
+    if (ok) PASS(name); else FAIL(name, "step=%d", moved.get_step());
+}
+
+// 5. clip: pre-clip norm returned, workspace tail included and scaled, fused == unfused
+static void test_clip() {
+    const char* name = "clip_grad_norm_ and fused clip";
+    const float max_norm = 0.25f;
+    Fixture a(5e-3f), b(5e-3f);
+    AdamWOptimizer oa(a.pools, 1e-3f, 0.9f, 0.999f, 1e-8f, 0.01f, /*use_master=*/false);
+    AdamWOptimizer ob(b.pools, 1e-3f, 0.9f, 0.999f, 1e-8f, 0.01f, /*use_master=*/false);
+    OptimStepConfig ca; ca.max_grad_norm = max_norm;
+    OptimStepConfig cb = ca; cb.fused_clip = true;
+    OptimStep sa(&oa, ca), sb(&ob, cb);
+    std::vector<uint16_t> og16 = a.h_g16;
+    std::vector<float> og32 = a.h_g32;
+    float o_scale = 0.0f;
+    float o_norm = orc_clip_grad_norm(og16.data(), a.n16, og32.data(), a.n32 + a.tail, max_norm, &o_scale);
+    float na = sa.apply(&a.grads), nb = sb.apply(&b.grads);
+    HIP_CHECK(hipDeviceSynchronize());
+    bool ok = na == nb && fabsf(na - o_norm) <= 1e-5f * o_norm && na > max_norm;
+    a.download(); b.download();
+    size_t bad_g = 0, untouched = 0, diff = 0;
+    for (size_t i = 0; i < a.n16; i++) { bad_g += a.h_g16[i] != og16[i]; diff += a.h_w16[i] != b.h_w16[i]; }
+    for (size_t i = 0; i < a.n32 + a.tail; i++) bad_g += memcmp(&a.h_g32[i], &og32[i], 4) != 0;
+    Fixture fresh(5e-3f);
+    for (size_t i = 0; i < b.n16; i++) untouched += b.h_g16[i] == fresh.h_g16[i];
+    for (size_t i = 0; i < a.n32; i++) diff += memcmp(&a.h_w32[i], &b.h_w32[i], 4) != 0;
+    double post = sqrt(orc_sum_sq_half(a.h_g16.data(), a.n16) + orc_sum_sq_float(a.h_g32.data(), a.n32 + a.tail));
+    printf("  norm=%.6f (oracle %.6f)  scaled-grad mismatches=%zu  fused-vs-unfused diffs=%zu  post-clip norm=%.6f\n",
+           na, o_norm, bad_g, diff, post);
+    ok = ok && bad_g == 0 && diff == 0 && untouched == b.n16 && post <= max_norm * 1.002;
+    if (ok) PASS(name); else FAIL(name, "na=%f nb=%f", na, nb);
+}
+
+// 6. operator API on raw pointers, n <= 0 no-op
+static void test_launch_api() {
+    const char* name = "launch_adamw_fp16 / launch_adamw_fp32";
+    Fixture f(1e-3f);
+    float *m, *v;
+    const int n = 10007;
+    HIP_CHECK(hipMalloc((void**)&m, n * 4)); HIP_CHECK(hipMalloc((void**)&v, n * 4));
+    HIP_CHECK(hipMemset(m, 0, n * 4)); HIP_CHECK(hipMemset(v, 0, n * 4));
+    launch_adamw_fp16(nullptr, f.w16, f.g16, m, v, 0, 1e-3f, 0.9f, 0.999f, 1e-8f, 0.01f, 0.1f, 0.001f);   // no-op
+    launch_adamw_fp16(nullptr, f.w16, f.g16, m, v, n, 1e-3f, 0.9f, 0.999f, 1e-8f, 0.01f, 0.1f, 0.001f);
+    HIP_CHECK(hipDeviceSynchronize());
+    std::vector<uint16_t> w = f.h_w16;
+    std::vector<float> om(n, 0.0f), ov(n, 0.0f);
+    orc_adamw_fp16(nullptr, w.data(), f.h_g16.data(), om.data(), ov.data(), n, 1e-3f, 0.9f, 0.999f, 1e-8f, 0.01f, 0.1f, 0.001f);
+    auto gw = d2h((const uint16_t*)f.w16, f.n16);
+    auto gm = d2h(m, n);
+    size_t bad = 0;
+    for (size_t i = 0; i < f.n16; i++) bad += gw[i] != w[i];
+    for (int i = 0; i < n; i++) bad += memcmp(&gm[i], &om[i], 4) != 0;
+    HIP_CHECK(hipMemset(m, 0, n * 4)); HIP_CHECK(hipMemset(v, 0, n * 4));
+    launch_adamw_fp32(f.w32, f.g32, m, v, (int)f.n32, 1e-3f, 0.9f, 0.999f, 1e-8f, 0.0f, 0.1f, 0.001f);
+    HIP_CHECK(hipDeviceSynchronize());
+    std::vector<float> w32 = f.h_w32, m32(f.n32, 0.0f), v32(f.n32, 0.0f);
+    orc_adamw_fp32(w32.data(), f.h_g32.data(), m32.data(), v32.data(), f.n32, 1e-3f, 0.9f, 0.999f, 1e-8f, 0.0f, 0.1f, 0.001f);
+    auto gw32 = d2h(f.w32, f.n32);
+    for (size_t i = 0; i < f.n32; i++) bad += memcmp(&gw32[i], &w32[i], 4) != 0;
+    (void)hipFree(m); (void)hipFree(v);
+    if (bad == 0) PASS(name); else FAIL(name, "%zu mismatches", bad);
+}
+
+int main() {
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
+        printf("no GPU: this test needs one\n");
+        return 2;
+    }
+    printf("=== AdamW host-side tests ===\n");
+    test_cpu_reference_fp32();
+    test_cpu_reference_fp16();
+    test_moments_nonzero();
+    test_step_counter();
+    test_clip();
+    test_launch_api();
+    printf("=== %s (%d failure%s) ===\n", g_fails ? "FAILED" : "ALL PASSED", g_fails, g_fails == 1 ? "" : "s");
+    return g_fails;
+}
