@@ -380,7 +380,16 @@ __global__ __launch_bounds__(kFinalBlock) void sumsq_final_kernel(
     __shared__ double acc[kFinalBlock];
     const int tid = threadIdx.x;
     double a = 0.0;
-    for (int64_t i = tid; i < n_partials; i += kFinalBlock) a += partials[i];
+    int64_t i = tid;
+    // eight independent loads in flight, added in index order: the same sum as one at a time
+    for (; i + 7 * (int64_t)kFinalBlock < n_partials; i += 8 * (int64_t)kFinalBlock) {
+        double x[8];
+#pragma unroll
+        for (int k = 0; k < 8; k++) x[k] = partials[i + k * (int64_t)kFinalBlock];
+#pragma unroll
+        for (int k = 0; k < 8; k++) a += x[k];
+    }
+    for (; i < n_partials; i += kFinalBlock) a += partials[i];
     acc[tid] = a;
     __syncthreads();
     for (int s = kFinalBlock / 2; s >= 1; s >>= 1) {
