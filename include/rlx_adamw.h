@@ -69,9 +69,16 @@ enum { RLX_DTYPE_F16 = 0, RLX_DTYPE_F32 = 1 };
 enum {
     RLX_TENSOR_NO_DECAY  = 1,   /* weight_decay is 0 for this tensor (embedding and norm
                                    groups, include/training/optimizer.h:131-146) */
-    RLX_TENSOR_GRAD_ONLY = 2    /* no parameter: the buffer only takes part in the norm and
+    RLX_TENSOR_GRAD_ONLY = 2,   /* no parameter: the buffer only takes part in the norm and
                                    in the scale pass (the D_buf tail of the reference's
                                    float_pool, include/training/trainer.h:330-337) */
+    RLX_TENSOR_FROZEN    = 4    /* the tensor's gradient counts as zero: it is neither read by
+                                   the norm nor scaled, and the update leaves p, m, v alone.
+                                   Equals what the reference does for a frozen embedding
+                                   (gradients cleared before the clip, then an identity
+                                   update; include/training/trainer.h:269-277,
+                                   optimizer.h:131-140) as long as the tensor's moments are
+                                   zero and it has no weight decay. */
 };
 
 typedef struct rlx_tensor_desc {
@@ -140,14 +147,28 @@ int rlx_plan_scale_grads(rlx_plan* plan, void* stream);
 /*
  * One AdamW step over every tensor of the plan in a single launch: replaces the three
  * launches of AdamWOptimizer::step (include/training/optimizer.h:124-146).
- * clip_mode: RLX_CLIP_NONE  gradients are used as stored;
- *            RLX_CLIP_FUSED the scale left by rlx_plan_grad_norm on the device is applied
- *                           to each gradient in registers (FP16 gradients re-rounded to
- *                           FP16 first, exactly as rlx_plan_scale_grads would have stored
- *                           them); the gradient buffers are not written.
+ * step_flags, any combination of:
+ *   RLX_CLIP_FUSED       the scale left by rlx_plan_grad_norm on the device is applied to each
+ *                        gradient in registers (FP16 gradients re-rounded to FP16 first, exactly
+ *                        as rlx_plan_scale_grads would have stored them); without
+ *                        RLX_STEP_ZERO_GRADS the gradient buffers are not written.
+ *   RLX_STEP_ZERO_GRADS  every gradient buffer of the plan (grad-only and frozen ones too) is
+ *                        cleared after it has been read: replaces the two memsets of
+ *                        qwen3_gradients_zero at the start of the next step
+ *                        (src/model/qwen3.cu:1109-1112, include/training/trainer.h:242).
+ * 0 (RLX_CLIP_NONE) uses the gradients as stored and leaves them alone.
  */
-enum { RLX_CLIP_NONE = 0, RLX_CLIP_FUSED = 1 };
-int rlx_plan_adamw(rlx_plan* plan, const rlx_step_params* params, int clip_mode, void* stream);
+enum { RLX_CLIP_NONE = 0, RLX_CLIP_FUSED = 1, RLX_STEP_ZERO_GRADS = 2 };
+int rlx_plan_adamw(rlx_plan* plan, const rlx_step_params* params, int step_flags, void* stream);
+
+/*
+ * The same step with the hyper-parameters read from device memory at run time (28 bytes,
+ * 4-byte aligned), so that a recorded launch (HIP graph) can be replayed with a new learning
+ * rate and new bias corrections: the host only rewrites *dev_params between replays.  No
+ * counterpart in the reference, whose step takes them by value (optimizer.h:119-147).
+ * The values are not validated.
+ */
+int rlx_plan_adamw_dev(rlx_plan* plan, const rlx_step_params* dev_params, int step_flags, void* stream);
 
 /* ------------------------------------------------------------------------------------
  * Launch tuning (process-wide; for measurement).  Unknown keys return RLX_ERR_INVALID_ARG.

@@ -12,8 +12,8 @@ LIB_PATH = os.path.join(HERE, "librlx_adamw.so")
 
 OK, ERR_INVALID_ARG, ERR_MISALIGNED, ERR_BAD_HYPER, ERR_HIP, ERR_NO_DEVICE, ERR_TOO_LARGE = range(7)
 DTYPE_F16, DTYPE_F32 = 0, 1
-TENSOR_NO_DECAY, TENSOR_GRAD_ONLY = 1, 2
-CLIP_NONE, CLIP_FUSED = 0, 1
+TENSOR_NO_DECAY, TENSOR_GRAD_ONLY, TENSOR_FROZEN = 1, 2, 4
+CLIP_NONE, CLIP_FUSED, STEP_ZERO_GRADS = 0, 1, 2
 FILL_ABS = 1
 
 
@@ -55,6 +55,7 @@ SIGNATURES = {
     "rlx_plan_partials_device_ptr": ([_VP], _VP),
     "rlx_plan_scale_grads": ([_VP, _VP], _INT),
     "rlx_plan_adamw": ([_VP, C.POINTER(StepParams), _INT, _VP], _INT),
+    "rlx_plan_adamw_dev": ([_VP, _VP, _INT, _VP], _INT),
     "rlx_set_tuning": ([C.c_char_p, _I64], _INT),
     "rlx_get_tuning": ([C.c_char_p], _I64),
     "rlx_fill_f16": ([_VP, _I64, _U64, _I64, _F, _F, _U32, _I64, _U32, _VP], _INT),
@@ -178,8 +179,11 @@ class Plan:
     def scale_grads(self, stream=0):
         check(load().rlx_plan_scale_grads(self._h, stream), "rlx_plan_scale_grads")
 
-    def adamw(self, params, clip_mode=CLIP_NONE, stream=0):
-        check(load().rlx_plan_adamw(self._h, C.byref(params), clip_mode, stream), "rlx_plan_adamw")
+    def adamw(self, params, step_flags=CLIP_NONE, stream=0):
+        check(load().rlx_plan_adamw(self._h, C.byref(params), step_flags, stream), "rlx_plan_adamw")
+
+    def adamw_dev(self, dev_params_ptr, step_flags=CLIP_NONE, stream=0):
+        check(load().rlx_plan_adamw_dev(self._h, dev_params_ptr, step_flags, stream), "rlx_plan_adamw_dev")
 
     def destroy(self):
         if self._h is not None:

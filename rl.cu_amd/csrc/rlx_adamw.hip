@@ -117,8 +117,18 @@ __device__ __forceinline__ void adamw_elem(float g, float& m, float& v, float& w
     w = w * (1.0f - h.lr * wd) - h.lr * m_hat / (__builtin_sqrtf(v_hat) + h.eps);
 }
 
-// Clip as a preceding scale pass would have stored it (trainer.h:136-139): re-round to FP16.
-__device__ __forceinline__ float clip_f16(float g, float scale) { return h2f(f2h(g * scale)); }
+// FP16 gradient times the clip scale, as scale_half_kernel stores it (trainer.h:136-139): the
+// product is rounded to FP32 and then to FP16.  Left to itself the compiler merges the multiply and
+// the conversion into one v_fma_mixlo_f16, which rounds the exact product once and differs in the
+// last FP16 bit for about one value in 10^4; the empty asm keeps the two roundings apart.
+__device__ __forceinline__ uint32_t scaled_f16_bits(float g, float scale) {
+    float t = g * scale;
+    asm volatile("" : "+v"(t));
+    return f2h(t);
+}
+
+// Clip as a preceding scale pass would have stored it: re-round to FP16, continue in FP32.
+__device__ __forceinline__ float clip_f16(float g, float scale) { return h2f(scaled_f16_bits(g, scale)); }
 
 // E packed FP16 values and E FP32 values as one access each.
 template <int E> struct Lane;
@@ -198,7 +208,8 @@ __device__ __forceinline__ void update_scalar32(const ChunkRec& r, int64_t i, co
 template <int E, int BLOCK, int K, bool SINGLE>
 __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
     const ChunkRec* __restrict__ recs, ChunkRec single, int64_t single_n, int64_t first_tile, int64_t n_tiles,
-    int tiles_per_chunk_log2, Hyper h, const NormResult* __restrict__ norm)
+    int tiles_per_chunk_log2, Hyper h, const rlx_step_params* __restrict__ dev_params,
+    const NormResult* __restrict__ norm, uint32_t step_flags)
 {
     constexpr int TILE = E * BLOCK;
     int64_t b = blockIdx.x;
@@ -221,26 +232,56 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         off = (tile & ((1 << tiles_per_chunk_log2) - 1)) * TILE;
         left = (int64_t)r.count - off;
     }
-    if (left <= 0 || (r.flags & RLX_TENSOR_GRAD_ONLY)) return;
+    if (left <= 0) return;
     const int n_here = left < TILE ? (int)left : TILE;
-    const bool clip = norm != nullptr;
-    const float scale = clip ? norm->scale : 1.0f;
-    const float wd = (r.flags & RLX_TENSOR_NO_DECAY) ? 0.0f : h.weight_decay;
     const bool is_f32 = (r.flags & kF32) != 0;
     const int valign = (r.flags >> kValignShift) & 0xF;
     const int e0 = threadIdx.x * E;
     const int64_t i0 = off + e0;
+    const bool zero_grads = (step_flags & RLX_STEP_ZERO_GRADS) != 0;
+    const bool vec = valign >= E && e0 + E <= n_here;
+    typedef typename Lane<E>::H HV;
+    typedef typename Lane<E>::F FV;
 
-    if (valign < E || e0 + E > n_here) {
-        for (int e = e0; e < e0 + E && e < n_here; e++) {
-            if (is_f32) update_scalar32(r, off + e, h, wd, scale, clip);
-            else update_scalar16(r, off + e, h, wd, scale, clip);
+    if (r.flags & (RLX_TENSOR_GRAD_ONLY | RLX_TENSOR_FROZEN)) {
+        // no update here; the buffer is only cleared for the next accumulation
+        if (zero_grads) {
+            if (vec) {
+                if (is_f32) stg<true>((FV*)((float*)r.g + i0), FV{});
+                else stg<true>((HV*)((uint16_t*)r.g + i0), HV{});
+            } else {
+                for (int e = e0; e < e0 + E && e < n_here; e++) {
+                    if (is_f32) stg<true>((float*)r.g + off + e, 0.0f);
+                    else stg<true>((uint16_t*)r.g + off + e, (uint16_t)0);
+                }
+            }
         }
         return;
     }
 
-    typedef typename Lane<E>::H HV;
-    typedef typename Lane<E>::F FV;
+    if (dev_params) {      // hyper-parameters resident on the device (replayable launches)
+        h.lr = dev_params->lr; h.beta1 = dev_params->beta1; h.beta2 = dev_params->beta2; h.eps = dev_params->eps;
+        h.weight_decay = dev_params->weight_decay;
+        h.bc1_inv = 1.0f / dev_params->bias_correction1;
+        h.bc2_inv = 1.0f / dev_params->bias_correction2;
+    }
+    const bool clip = norm != nullptr;
+    const float scale = clip ? norm->scale : 1.0f;
+    const float wd = (r.flags & RLX_TENSOR_NO_DECAY) ? 0.0f : h.weight_decay;
+
+    if (!vec) {
+        for (int e = e0; e < e0 + E && e < n_here; e++) {
+            if (is_f32) {
+                update_scalar32(r, off + e, h, wd, scale, clip);
+                if (zero_grads) stg<true>((float*)r.g + off + e, 0.0f);
+            } else {
+                update_scalar16(r, off + e, h, wd, scale, clip);
+                if (zero_grads) stg<true>((uint16_t*)r.g + off + e, (uint16_t)0);
+            }
+        }
+        return;
+    }
+
     float g[E], m[E], v[E], w[E];
     if (!is_f32) {
         const bool has_master = r.master != nullptr;
@@ -262,6 +303,7 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         stg<true>((FV*)(r.v + i0), pack_f<E>(v));
         if (has_master) stg<true>((FV*)(r.master + i0), pack_f<E>(w));
         stg<true>((HV*)((uint16_t*)r.p + i0), pack_h<E>(w));
+        if (zero_grads) stg<true>((HV*)((uint16_t*)r.g + i0), HV{});
     } else {
         // FP32 parameters (norm weights): the same update, in place (adamw.cu:80-90)
         unpack_f<E>(ldg<true>((const FV*)((const float*)r.g + i0)), g);
@@ -277,6 +319,7 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         stg<true>((FV*)(r.m + i0), pack_f<E>(m));
         stg<true>((FV*)(r.v + i0), pack_f<E>(v));
         stg<true>((FV*)((float*)r.p + i0), pack_f<E>(w));
+        if (zero_grads) stg<true>((FV*)((float*)r.g + i0), FV{});
     }
 }
 
@@ -301,7 +344,9 @@ __global__ __launch_bounds__(kNormBlock) void sumsq_partials_kernel(
         const bool aligned = ((r.flags >> kValignShift) & 0xF) >= 8;
 
         float acc = 0.0f;
-        if (!(r.flags & kF32)) {
+        if (r.flags & RLX_TENSOR_FROZEN) {
+            // gradients of a frozen tensor count as zero (the reference clears them before the norm)
+        } else if (!(r.flags & kF32)) {
             const uint16_t* g = (const uint16_t*)r.g;
             int64_t done = 0;
             if (aligned) {
@@ -416,6 +461,7 @@ __global__ __launch_bounds__(kNormBlock) void scale_grads_kernel(
     const int tid = threadIdx.x;
     for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
         const ChunkRec r = recs[c];
+        if (r.flags & RLX_TENSOR_FROZEN) continue;
         const int64_t count = r.count;
         const bool aligned = ((r.flags >> kValignShift) & 0xF) >= 8;
         if (!(r.flags & kF32)) {
@@ -426,11 +472,11 @@ __global__ __launch_bounds__(kNormBlock) void scale_grads_kernel(
                     u32x4 x = ldg<true>((const u32x4*)(g + off));
 #pragma unroll
                     for (int k = 0; k < 4; k++)
-                        x[k] = f2h(h2f(x[k] & 0xFFFFu) * scale) | (f2h(h2f(x[k] >> 16) * scale) << 16);
+                        x[k] = scaled_f16_bits(h2f(x[k] & 0xFFFFu), scale) | (scaled_f16_bits(h2f(x[k] >> 16), scale) << 16);
                     stg<true>((u32x4*)(g + off), x);
                 } else {
                     for (int64_t i = off; i < off + kVec && i < count; i++)
-                        g[i] = (uint16_t)f2h(h2f(g[i]) * scale);
+                        g[i] = (uint16_t)scaled_f16_bits(h2f(g[i]), scale);
                 }
             }
         } else {
@@ -543,7 +589,7 @@ Hyper make_hyper(float lr, float beta1, float beta2, float eps, float wd, float 
 int check_desc(const rlx_tensor_desc& d) {
     if (d.n <= 0 || !d.grad) return RLX_ERR_INVALID_ARG;
     if (d.dtype != RLX_DTYPE_F16 && d.dtype != RLX_DTYPE_F32) return RLX_ERR_INVALID_ARG;
-    if (d.flags & ~(uint32_t)(RLX_TENSOR_NO_DECAY | RLX_TENSOR_GRAD_ONLY)) return RLX_ERR_INVALID_ARG;
+    if (d.flags & ~(uint32_t)(RLX_TENSOR_NO_DECAY | RLX_TENSOR_GRAD_ONLY | RLX_TENSOR_FROZEN)) return RLX_ERR_INVALID_ARG;
     const bool grad_only = (d.flags & RLX_TENSOR_GRAD_ONLY) != 0;
     if (!grad_only && (!d.param || !d.m || !d.v)) return RLX_ERR_INVALID_ARG;
     if (d.master && d.dtype != RLX_DTYPE_F16) return RLX_ERR_INVALID_ARG;
@@ -582,7 +628,8 @@ struct UpdateVariant { int tile; };
 
 template <int E, int BLOCK, int K, bool SINGLE>
 void launch_variant(const ChunkRec* recs, const ChunkRec& single, int64_t single_n, int64_t n_elems_or_tiles,
-                    int chunk_log2, const Hyper& h, const NormResult* norm, hipStream_t s) {
+                    int chunk_log2, const Hyper& h, const rlx_step_params* dev_params, const NormResult* norm,
+                    uint32_t step_flags, hipStream_t s) {
     constexpr int TILE = E * BLOCK;
     int64_t n_tiles;
     int tpc_log2 = 0;
@@ -596,23 +643,24 @@ void launch_variant(const ChunkRec* recs, const ChunkRec& single, int64_t single
         int64_t here = n_tiles - first < kMaxTilesPerLaunch ? n_tiles - first : kMaxTilesPerLaunch;
         here = (here + 8 * K - 1) / (8 * K) * (8 * K);   // whole swizzle groups; the excess exits at once
         adamw_tile_kernel<E, BLOCK, K, SINGLE><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(
-            recs, single, single_n, first, n_tiles, tpc_log2, h, norm);
+            recs, single, single_n, first, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
     }
 }
 
 template <bool SINGLE>
 int launch_update(const ChunkRec* recs, const ChunkRec& single, int64_t single_n, int64_t n, int chunk_log2,
-                  const Hyper& h, const NormResult* norm, hipStream_t s) {
+                  const Hyper& h, const rlx_step_params* dev_params, const NormResult* norm, uint32_t step_flags,
+                  hipStream_t s) {
     switch (g_tuning.update_variant) {
     default:
-    case 0: launch_variant<2, 128, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
-    case 1: launch_variant<2, 128, 2, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
-    case 2: launch_variant<2, 64, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
-    case 3: launch_variant<2, 64, 2, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
-    case 4: launch_variant<4, 64, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
-    case 5: launch_variant<2, 256, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
-    case 6: launch_variant<1, 256, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
-    case 7: launch_variant<4, 128, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, norm, s); break;
+    case 0: launch_variant<2, 128, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 1: launch_variant<2, 128, 2, SINGLE>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 2: launch_variant<2, 64, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 3: launch_variant<2, 64, 2, SINGLE>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 4: launch_variant<4, 64, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 5: launch_variant<2, 256, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 6: launch_variant<1, 256, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 7: launch_variant<4, 128, 1, SINGLE>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
     }
     RLX_HIP(hipGetLastError());
     return RLX_OK;
@@ -630,8 +678,8 @@ int flat_update(void* p, const void* g, float* m, float* v, float* master, int64
     st = check_hyper(lr, beta1, beta2, eps, wd, bc1, bc2);
     if (st != RLX_OK) return st;
     const ChunkRec r = make_rec(d, 0, 0);
-    return launch_update<true>(nullptr, r, n, n, 0, make_hyper(lr, beta1, beta2, eps, wd, bc1, bc2), nullptr,
-                               (hipStream_t)stream);
+    return launch_update<true>(nullptr, r, n, n, 0, make_hyper(lr, beta1, beta2, eps, wd, bc1, bc2), nullptr, nullptr,
+                               0, (hipStream_t)stream);
 }
 
 }  // namespace
@@ -669,7 +717,7 @@ const char* rlx_status_string(int status) {
 
 const char* rlx_last_hip_error(void) { return g_hip_error; }
 
-int rlx_version(void) { return 100; }
+int rlx_version(void) { return 101; }
 
 int rlx_adamw_fp16(float* master_w, uint16_t* model_w, const uint16_t* grad, float* m, float* v, int64_t n,
                    float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -807,9 +855,9 @@ int rlx_plan_scale_grads(rlx_plan* p, void* stream) {
     return RLX_OK;
 }
 
-int rlx_plan_adamw(rlx_plan* p, const rlx_step_params* sp, int clip_mode, void* stream) {
+int rlx_plan_adamw(rlx_plan* p, const rlx_step_params* sp, int step_flags, void* stream) {
     if (!plan_ok(p) || !sp) return RLX_ERR_INVALID_ARG;
-    if (clip_mode != RLX_CLIP_NONE && clip_mode != RLX_CLIP_FUSED) return RLX_ERR_INVALID_ARG;
+    if (step_flags & ~(RLX_CLIP_FUSED | RLX_STEP_ZERO_GRADS)) return RLX_ERR_INVALID_ARG;
     int st = check_hyper(sp->lr, sp->beta1, sp->beta2, sp->eps, sp->weight_decay, sp->bias_correction1,
                          sp->bias_correction2);
     if (st != RLX_OK) return st;
@@ -817,8 +865,22 @@ int rlx_plan_adamw(rlx_plan* p, const rlx_step_params* sp, int clip_mode, void* 
                                sp->bias_correction2);
     ChunkRec none;
     memset(&none, 0, sizeof(none));
-    return launch_update<false>(p->d_recs, none, 0, p->n_chunks, p->chunk_log2, h,
-                                clip_mode == RLX_CLIP_FUSED ? p->d_norm : nullptr, (hipStream_t)stream);
+    return launch_update<false>(p->d_recs, none, 0, p->n_chunks, p->chunk_log2, h, nullptr,
+                                (step_flags & RLX_CLIP_FUSED) ? p->d_norm : nullptr, (uint32_t)step_flags,
+                                (hipStream_t)stream);
+}
+
+int rlx_plan_adamw_dev(rlx_plan* p, const rlx_step_params* dev_params, int step_flags, void* stream) {
+    if (!plan_ok(p) || !dev_params) return RLX_ERR_INVALID_ARG;
+    if (step_flags & ~(RLX_CLIP_FUSED | RLX_STEP_ZERO_GRADS)) return RLX_ERR_INVALID_ARG;
+    if (!is_aligned(dev_params, 4)) return RLX_ERR_MISALIGNED;
+    ChunkRec none;
+    memset(&none, 0, sizeof(none));
+    Hyper h;
+    memset(&h, 0, sizeof(h));
+    return launch_update<false>(p->d_recs, none, 0, p->n_chunks, p->chunk_log2, h, dev_params,
+                                (step_flags & RLX_CLIP_FUSED) ? p->d_norm : nullptr, (uint32_t)step_flags,
+                                (hipStream_t)stream);
 }
 
 int rlx_set_tuning(const char* key, int64_t value) {

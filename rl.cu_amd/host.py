@@ -143,12 +143,13 @@ class AdamWOptimizer:
         return B.StepParams(self.lr, self.beta1, self.beta2, self.eps, self.weight_decay,
                             bias_correction(self.beta1, self.step_), bias_correction(self.beta2, self.step_))
 
-    def step(self, fused_clip=False, stream=None):
+    def step(self, fused_clip=False, zero_grads=False, stream=None):
         """One launch over every tensor.  fused_clip: apply the scale that the last
-        clip_grad_norm_(..., fused=True) left on the device."""
+        clip_grad_norm_(..., fused=True) left on the device.  zero_grads: clear every gradient
+        buffer after it has been read (instead of qwen3_gradients_zero at the next step)."""
         self.step_ += 1
-        self.plan.adamw(self.step_params(), B.CLIP_FUSED if fused_clip else B.CLIP_NONE,
-                        _stream() if stream is None else stream)
+        flags = (B.CLIP_FUSED if fused_clip else 0) | (B.STEP_ZERO_GRADS if zero_grads else 0)
+        self.plan.adamw(self.step_params(), flags, _stream() if stream is None else stream)
 
     def clip_grad_norm_(self, max_norm, fused=False, stream=None):
         """Returns the pre-clip norm (blocking read, as in the reference).  fused=False scales the
@@ -162,12 +163,12 @@ class AdamWOptimizer:
         return norm
 
 
-def training_step(optimizer, max_grad_norm, fused_clip=False):
+def training_step(optimizer, max_grad_norm, fused_clip=False, zero_grads=False):
     """The tail of Trainer::training_step (trainer.h:279-288): clip if max_grad_norm > 0, then step.
     Returns the pre-clip norm (0 if clipping is off)."""
     grad_norm = 0.0
     clipped = max_grad_norm > 0.0
     if clipped:
         grad_norm = optimizer.clip_grad_norm_(max_grad_norm, fused=fused_clip)
-    optimizer.step(fused_clip=fused_clip and clipped)
+    optimizer.step(fused_clip=fused_clip and clipped, zero_grads=zero_grads)
     return grad_norm

@@ -85,15 +85,27 @@ public:
     size_t num_fp16_params() const { return n16_; }
     size_t num_fp32_params() const { return n32_; }
 
+    // Treat the embedding (the tail of the FP16 pool) as frozen: its gradients count as zero in the
+    // norm and the update leaves it alone, instead of clearing the gradients and streaming an
+    // identity update over it (trainer.h:269-277).  Exact while its moments are zero.
+    void set_embed_frozen(bool frozen) {
+        if (frozen != embed_frozen_) {
+            embed_frozen_ = frozen;
+            if (plan_) { RLX_CHECK(rlx_plan_destroy(plan_)); plan_ = nullptr; }
+        }
+    }
+
     // One optimizer step.  fused_clip: apply the clip scale that the last norm pass of
-    // plan_for(grads) left on the device, inside the update (gradients are not written).
-    void step(GradPools* grads, hipStream_t stream = 0, bool fused_clip = false) {
+    // plan_for(grads) left on the device, inside the update.  zero_grads: clear both gradient
+    // pools after they have been read (the job of qwen3_gradients_zero at the next step).
+    void step(GradPools* grads, hipStream_t stream = 0, bool fused_clip = false, bool zero_grads = false) {
         step_++;
         rlx_step_params sp;
         sp.lr = lr; sp.beta1 = beta1; sp.beta2 = beta2; sp.eps = eps; sp.weight_decay = weight_decay;
         sp.bias_correction1 = 1.0f - powf(beta1, (float)step_);
         sp.bias_correction2 = 1.0f - powf(beta2, (float)step_);
-        RLX_CHECK(rlx_plan_adamw(plan_for(grads), &sp, fused_clip ? RLX_CLIP_FUSED : RLX_CLIP_NONE, (void*)stream));
+        const int flags = (fused_clip ? RLX_CLIP_FUSED : 0) | (zero_grads ? RLX_STEP_ZERO_GRADS : 0);
+        RLX_CHECK(rlx_plan_adamw(plan_for(grads), &sp, flags, (void*)stream));
     }
 
     // The multi-tensor plan over {projections, embedding, norm weights, workspace tail} for these
@@ -115,7 +127,7 @@ public:
         if (embed_n) {   // no decay on the embedding (optimizer.h:131-140)
             d[k++] = {pools_.fp16_pool + proj_n_, grads->half_pool + proj_n_, fp16_m_ + proj_n_, fp16_v_ + proj_n_,
                       fp16_master_ ? fp16_master_ + proj_n_ : nullptr, (int64_t)embed_n, RLX_DTYPE_F16,
-                      RLX_TENSOR_NO_DECAY};
+                      (uint32_t)(RLX_TENSOR_NO_DECAY | (embed_frozen_ ? RLX_TENSOR_FROZEN : 0))};
         }
         if (n32_) {      // no decay on the norm weights (optimizer.h:142-146)
             d[k++] = {pools_.fp32_pool, grads->float_pool, fp32_m_, fp32_v_, nullptr, (int64_t)n32_, RLX_DTYPE_F32,
@@ -146,6 +158,7 @@ private:
     half* plan_half_ = nullptr;
     float* plan_float_ = nullptr;
     size_t plan_float_bytes_ = 0;
+    bool embed_frozen_ = false;
 
     void init(const ParamPools& pools, bool use_master) {
         pools_ = pools;
@@ -194,6 +207,7 @@ private:
         fp16_state_ = o.fp16_state_; fp32_state_ = o.fp32_state_;
         n16_ = o.n16_; n32_ = o.n32_; proj_n_ = o.proj_n_;
         plan_ = o.plan_; plan_half_ = o.plan_half_; plan_float_ = o.plan_float_; plan_float_bytes_ = o.plan_float_bytes_;
+        embed_frozen_ = o.embed_frozen_;
         o.plan_ = nullptr; o.fp16_state_ = nullptr; o.fp32_state_ = nullptr;
         o.fp16_master_ = o.fp16_m_ = o.fp16_v_ = o.fp32_m_ = o.fp32_v_ = nullptr;
     }

@@ -8,6 +8,10 @@ struct OptimStepConfig {          // the fields of TrainingConfig that this path
     float max_grad_norm = 1.0f;   // <= 0 disables clipping
     bool freeze_embed = false;
     bool fused_clip = false;      // apply the clip scale inside the update instead of a scale pass
+    bool zero_grads = false;      // clear the gradient pools inside the update (then the caller drops its
+                                  // qwen3_gradients_zero at the start of the next step)
+    bool freeze_in_plan = false;  // with freeze_embed: flag the embedding as frozen in the plan instead
+                                  // of clearing its gradients and updating it with zeros
 };
 
 class OptimStep {
@@ -28,7 +32,8 @@ public:
     // What training_step does after the backward passes.  embed_elems: size of the embedding at
     // the end of half_pool (only read when freeze_embed is set).  Returns the pre-clip norm.
     float apply(GradPools* grads, size_t embed_elems = 0, hipStream_t stream = 0) {
-        if (config_.freeze_embed && embed_elems) {
+        optimizer_->set_embed_frozen(config_.freeze_embed && config_.freeze_in_plan);
+        if (config_.freeze_embed && !config_.freeze_in_plan && embed_elems) {
             const size_t half_elems = grads->half_pool_bytes / sizeof(half);
             half* embed_grad = grads->half_pool + (half_elems - embed_elems);
             // zeros through a fill kernel (0 + 0 * z), which unlike a memset node is safe to capture
@@ -38,7 +43,7 @@ public:
         float grad_norm = 0.0f;
         const bool clip = config_.max_grad_norm > 0.0f;
         if (clip) grad_norm = clip_grad_norm_(grads, config_.max_grad_norm, stream);
-        optimizer_->step(grads, stream, clip && config_.fused_clip);
+        optimizer_->step(grads, stream, clip && config_.fused_clip, config_.zero_grads);
         last_grad_norm_ = grad_norm;
         return grad_norm;
     }

@@ -9,6 +9,7 @@ from collections import namedtuple
 
 DTYPE_F16, DTYPE_F32 = 0, 1
 NO_DECAY = 1
+FROZEN = 4
 
 # n elements; row_len > 0 marks a 2-D tensor whose rows can be masked (embedding)
 TensorSpec = namedtuple("TensorSpec", "name n dtype flags row_len")
@@ -19,13 +20,15 @@ QWEN3_8B = dict(vocab=151936, hidden=4096, inter=12288, layers=36, q_heads=32, k
                 tied=False)
 
 
-def qwen3_tensor_list(cfg, norm_dtype=DTYPE_F16, reference_decay_groups=False):
+def qwen3_tensor_list(cfg, norm_dtype=DTYPE_F16, reference_decay_groups=False, freeze_embed=False):
     """All parameter tensors of a Qwen3 model.
 
     norm_dtype: DTYPE_F16 keeps every tensor FP16 (the benchmark configurations);
     DTYPE_F32 gives the reference's layout, where norm weights and their gradients are FP32.
     reference_decay_groups: embedding and norm tensors get NO_DECAY, as the reference's
     step does (include/training/optimizer.h:131-146); otherwise every tensor decays.
+    freeze_embed: the embedding is marked FROZEN (TrainingConfig::freeze_embed,
+    include/training/trainer.h:269-277; the SFT main sets it).
     """
     H, I = cfg["hidden"], cfg["inter"]
     q_dim, kv_dim, hd = cfg["q_heads"] * cfg["head_dim"], cfg["kv_heads"] * cfg["head_dim"], cfg["head_dim"]
@@ -43,7 +46,7 @@ def qwen3_tensor_list(cfg, norm_dtype=DTYPE_F16, reference_decay_groups=False):
                   TensorSpec("layers.%d.q_norm" % l, hd, norm_dtype, nd, 0),
                   TensorSpec("layers.%d.k_norm" % l, hd, norm_dtype, nd, 0),
                   TensorSpec("layers.%d.post_attn_norm" % l, H, norm_dtype, nd, 0)]
-    embed = [TensorSpec("embed_tokens", cfg["vocab"] * H, DTYPE_F16, nd, H)]
+    embed = [TensorSpec("embed_tokens", cfg["vocab"] * H, DTYPE_F16, nd | (FROZEN if freeze_embed else 0), H)]
     if not cfg["tied"]:
         embed.append(TensorSpec("lm_head", cfg["vocab"] * H, DTYPE_F16, 0, H))
     norms.append(TensorSpec("final_norm", H, norm_dtype, nd, 0))

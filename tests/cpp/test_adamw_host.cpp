@@ -9,6 +9,7 @@
 //   4. get_step() counts 0 -> 3
 //   5. clip_grad_norm_ returns the pre-clip norm; clipped gradients have norm <= max; fused == unfused
 //   6. operator API (launch_adamw_fp16 / launch_adamw_fp32) on raw pointers
+//   7. frozen embedding flagged in the plan, gradients cleared inside the update
 // The oracle (liborc_adamw.so) is used as the checker only.
 #include <cmath>
 #include <cstdint>
@@ -235,6 +236,30 @@ static void test_launch_api() {
     if (bad == 0) PASS(name); else FAIL(name, "%zu mismatches", bad);
 }
 
+// 7. frozen embedding in the plan + gradient clearing inside the update == memset + identity update
+static void test_frozen_and_zeroing() {
+    const char* name = "frozen embedding and zeroing in the update";
+    Fixture a(5e-3f), b(5e-3f);
+    AdamWOptimizer oa(a.pools, 1e-3f), ob(b.pools, 1e-3f);
+    OptimStepConfig ca; ca.max_grad_norm = 0.25f; ca.freeze_embed = true; ca.fused_clip = true;
+    OptimStepConfig cb = ca; cb.freeze_in_plan = true; cb.zero_grads = true;
+    OptimStep sa(&oa, ca), sb(&ob, cb);
+    float na = sa.apply(&a.grads, a.embed_n), nb = sb.apply(&b.grads, b.embed_n);
+    HIP_CHECK(hipDeviceSynchronize());
+    std::vector<uint16_t> w0 = a.h_w16;
+    a.download(); b.download();
+    size_t diff = 0, nonzero = 0, moved = 0;
+    for (size_t i = 0; i < a.n16; i++) diff += a.h_w16[i] != b.h_w16[i];
+    for (size_t i = 0; i < a.n32; i++) diff += memcmp(&a.h_w32[i], &b.h_w32[i], 4) != 0;
+    for (size_t i = a.proj_n; i < a.n16; i++) moved += a.h_w16[i] != w0[i];
+    for (uint16_t x : b.h_g16) nonzero += x != 0;
+    for (float x : b.h_g32) nonzero += x != 0.0f;
+    auto ma = d2h(oa.fp16_m(), a.n16), mb = d2h(ob.fp16_m(), b.n16);
+    for (size_t i = 0; i < a.n16; i++) diff += memcmp(&ma[i], &mb[i], 4) != 0;
+    printf("  norm %.6f / %.6f  diffs=%zu  embedding weights moved=%zu  gradients left=%zu\n", na, nb, diff, moved, nonzero);
+    if (na == nb && diff == 0 && moved == 0 && nonzero == 0) PASS(name); else FAIL(name, "diff=%zu", diff);
+}
+
 int main() {
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
@@ -248,6 +273,7 @@ int main() {
     test_step_counter();
     test_clip();
     test_launch_api();
+    test_frozen_and_zeroing();
     printf("=== %s (%d failure%s) ===\n", g_fails ? "FAILED" : "ALL PASSED", g_fails, g_fails == 1 ? "" : "s");
     return g_fails;
 }

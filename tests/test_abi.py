@@ -39,7 +39,7 @@ def test_struct_layouts_match(B):
 
 def test_version_and_status_strings(B):
     lib = B.load()
-    assert lib.rlx_version() == 100
+    assert lib.rlx_version() >= 100
     assert lib.rlx_status_string(B.OK) == b"ok"
     for st in range(1, 7):
         assert lib.rlx_status_string(st) not in (b"ok", b"unknown status")
@@ -86,6 +86,7 @@ def test_plan_argument_checks(B):
     assert lib.rlx_plan_num_chunks(None) == -1
     assert lib.rlx_plan_grad_norm(None, 1.0, None) == B.ERR_INVALID_ARG
     assert lib.rlx_plan_adamw(None, None, 0, None) == B.ERR_INVALID_ARG
+    assert lib.rlx_plan_adamw_dev(None, None, 0, None) == B.ERR_INVALID_ARG
 
 
 def test_tuning_keys(B):

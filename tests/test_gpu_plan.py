@@ -272,3 +272,137 @@ def test_unaligned_tensors_in_a_plan(O, L, host, B, torch_gpu):
                  sp.bias_correction2, clip_scale=scale)
     assert np.array_equal(bits(pool_p), hp) and np.array_equal(bits(pool_m), hm) and np.array_equal(bits(pool_v), hv)
     plan.destroy()
+
+
+def test_zero_grads_in_the_update_and_frozen_embedding(O, L, host, B, torch_gpu):
+    """The reference's step is: clear all gradients (qwen3.cu:1109-1112), accumulate, clear the frozen
+    embedding's gradients (trainer.h:269-277), clip, update.  Here the frozen tensor is flagged in the
+    plan and the update clears every gradient buffer after reading it.  Weights, moments and the norm
+    must come out as in the reference's order of operations, and all gradient buffers must be zero."""
+    torch = torch_gpu
+    ref_specs = L.qwen3_tensor_list(MINI, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
+    frz_specs = L.qwen3_tensor_list(MINI, norm_dtype=L.DTYPE_F32, reference_decay_groups=True, freeze_embed=True)
+    emb = [i for i, s in enumerate(ref_specs) if s.name == "embed_tokens"][0]
+    assert frz_specs[emb].flags & L.FROZEN
+    st_a, st_b = host.ParamStore(ref_specs), host.ParamStore(frz_specs)
+    tails = [torch.empty(555, dtype=torch.float32, device="cuda:0") for _ in range(2)]
+    opt_a = host.AdamWOptimizer(st_a, lr=1e-3, chunk_elems=2048, extra_grad_only=(tails[0],))
+    opt_b = host.AdamWOptimizer(st_b, lr=1e-3, chunk_elems=2048, extra_grad_only=(tails[1],))
+    for st in (st_a, st_b):
+        st.fill("p", 1, 0.0, 0.02)
+    torch.cuda.synchronize()
+    hs = host_copy(st_a)
+    for step in range(1, 4):
+        for st, tail in ((st_a, tails[0]), (st_b, tails[1])):
+            st.fill("g", 50 + step, 0.0, 5e-3)
+            B.fill_f32(tail.data_ptr(), 555, 60 + step, 0.0, 0.1)
+        st_a.grad(emb).zero_()                                   # the reference's freeze_embed memset
+        torch.cuda.synchronize()
+        for i, h in enumerate(hs):
+            h["g"] = bits(st_a.grad(i))
+        tail_h = bits(tails[0])
+        na = host.training_step(opt_a, 0.5, fused_clip=True)
+        nb = host.training_step(opt_b, 0.5, fused_clip=True, zero_grads=True)
+        torch.cuda.synchronize()
+        assert na == nb and na > 0.5
+        _, scale, _ = opt_b.plan.norm_read()
+        oracle_step(O, L, ref_specs, hs, step, dict(HYPER, lr=1e-3), clip_scale=scale)
+        assert compare(st_a, hs, "reference order, step %d" % step) == 0
+        assert compare(st_b, hs, "frozen + zeroing, step %d" % step) == 0
+        assert not st_b.g16.any().item() and not st_b.g32.any().item() and not tails[1].any().item()
+        assert np.array_equal(bits(tails[0]), tail_h)            # without the flag nothing is cleared
+    assert not st_b.state(emb, "m").any().item() and not st_b.state(emb, "v").any().item()
+
+
+def test_device_resident_step_params_and_graph_replay(O, L, host, B, torch_gpu):
+    """norm + fused-clip update recorded once as a HIP graph and replayed for several steps; between
+    replays the host rewrites the 28 bytes of hyper-parameters on the device and new gradients arrive.
+    Every replay is checked against the oracle, with eager work and synchronisations in between."""
+    import ctypes as C
+    torch = torch_gpu
+    specs = L.qwen3_tensor_list(MINI, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
+    st = host.ParamStore(specs)
+    st.fill("p", 1, 0.0, 0.02)
+    st.fill("g", 2, 0.0, 5e-3)
+    opt = host.AdamWOptimizer(st, lr=1e-3, chunk_elems=2048)
+    torch.cuda.synchronize()
+    hs = host_copy(st)
+    dev_params = torch.zeros(7, dtype=torch.float32, device="cuda:0")
+    pinned = torch.zeros(7, dtype=torch.float32).pin_memory()
+
+    def set_params(step, lr):
+        sp = B.StepParams(lr, 0.9, 0.999, 1e-8, 0.01, host.bias_correction(0.9, step),
+                          host.bias_correction(0.999, step))
+        pinned.copy_(torch.frombuffer(bytearray(bytes(sp)), dtype=torch.float32))
+        dev_params.copy_(pinned, non_blocking=True)
+
+    side = torch.cuda.Stream()
+    set_params(1, 1e-3)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        # warm-up launch outside capture, on a throw-away copy of nothing: the kernels need no lazy init,
+        # but torch wants the capture stream used once
+        torch.cuda.synchronize()
+        with torch.cuda.graph(graph, stream=side):
+            s = torch.cuda.current_stream().cuda_stream
+            opt.plan.grad_norm(0.5, s)
+            opt.plan.adamw_dev(dev_params.data_ptr(), B.CLIP_FUSED, s)
+    torch.cuda.synchronize()
+    for step in range(1, 6):
+        lr = 1e-3 / step
+        if step > 1:
+            st.fill("g", 2 + step, 0.0, 5e-3 * step)             # eager work between replays
+            torch.cuda.synchronize()
+            for i, h in enumerate(hs):
+                h["g"] = bits(st.grad(i))
+        set_params(step, lr)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        norm, scale, sum_sq = opt.plan.norm_read()
+        truth = sum(O.sum_sq_half(h["g"]) if h["g"].dtype == np.uint16 else O.sum_sq_float(h["g"]) for h in hs)
+        assert abs(sum_sq - truth) <= 1e-5 * truth and norm > 0.5
+        assert sum_sq == O.sumsq_mirror([h["g"] for h in hs], 2048)[0]
+        oracle_step(O, L, specs, hs, step, dict(HYPER, lr=lr), clip_scale=scale)
+        assert compare(st, hs, "replay %d" % step) == 0
+    del C
+
+
+def test_clip_rounds_twice_for_every_half_and_many_scales(O, L, host, B, torch_gpu):
+    """g' = f2h(h2f(g) * scale) rounds the product to FP32 and then to FP16 (trainer.h:136-139).  A fused
+    multiply-convert rounds once and differs in the last bit for about one value in 10^4, and only for
+    scales with a full mantissa, so this walks every FP16 value of magnitude <= 2 under 48 different
+    scales, through the scale pass and through the fused update (the check at the end makes sure that the scales met
+    do tell one rounding from two)."""
+    torch = torch_gpu
+    pos = np.arange(0, 0x4001, dtype=np.uint32).astype(np.uint16)            # 0 .. 2.0
+    vals = np.concatenate([pos, pos | 0x8000])
+    n = vals.size
+    specs = [L.TensorSpec("all_halves", n, L.DTYPE_F16, 0, 0)]
+    mismatches_if_fused = 0
+    for k in range(48):
+        max_norm = 0.0123 * (1.19 ** k)
+        st = host.ParamStore(specs)
+        st.g16[:n].copy_(torch.from_numpy(vals.view(np.int16)).view(torch.float16))
+        st.fill("p", 1, 0.0, 0.02)
+        opt = host.AdamWOptimizer(st, lr=1e-3)
+        torch.cuda.synchronize()
+        hp = bits(st.param(0))
+        norm = host.training_step(opt, max_norm, fused_clip=True)
+        _, scale, _ = opt.plan.norm_read()
+        assert norm > max_norm and 0 < scale < 1
+        hm, hv = np.zeros(n, np.float32), np.zeros(n, np.float32)
+        O.adamw_fp16(None, hp, vals.copy(), hm, hv, 1e-3, 0.9, 0.999, 1e-8, 0.01, host.bias_correction(0.9, 1),
+                     host.bias_correction(0.999, 1), clip_scale=scale)
+        assert np.array_equal(bits(st.state(0, "m")), hm) and np.array_equal(bits(st.state(0, "v")), hv)
+        assert np.array_equal(bits(st.param(0)), hp)
+        opt.plan.scale_grads()
+        torch.cuda.synchronize()
+        want = vals.copy()
+        O.scale_half(want, scale)
+        assert np.array_equal(bits(st.grad(0)), want), "scale pass, max_norm %g" % max_norm
+        with np.errstate(all="ignore"):
+            once = (O.h2f(vals).astype(np.float64) * np.float64(np.float32(scale))).astype(np.float16).view(np.uint16)
+        mismatches_if_fused += int((once != want).sum())
+    assert mismatches_if_fused >= 3, "the scales chosen would not have told one rounding from two"
