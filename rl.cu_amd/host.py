@@ -9,6 +9,11 @@ torch is used for device memory and streams only; all arithmetic on tensors happ
 librlx_adamw.so.
 """
 import ctypes as C
+import json
+import math
+import os
+import struct
+import time
 
 from . import binding as B
 from .layout import DTYPE_F16, DTYPE_F32, _hash64
@@ -22,6 +27,40 @@ def bias_correction(beta, step):
     """1 - powf(beta, (float)step), in FP32 as on the reference's host (optimizer.h:121-122)."""
     import numpy as np
     return float(np.float32(1.0) - np.float32(_libm.powf(beta, float(step))))
+
+
+_libm.cosf.argtypes = [C.c_float]
+_libm.cosf.restype = C.c_float
+
+
+class LRScheduler:
+    """Warm-up, then constant or cosine decay: the reference's LRScheduler
+    (include/training/lr_scheduler.h:10-57) with the same methods, in FP32 step by step."""
+
+    def __init__(self):
+        self._cosine, self._base, self._min, self._warmup, self._total = False, 1e-5, 0.0, 0, 0
+
+    def init_constant(self, base_lr, warmup_steps=0):
+        self._cosine, self._base, self._min, self._warmup, self._total = False, base_lr, base_lr, warmup_steps, 0
+
+    def init_cosine(self, base_lr, min_lr, warmup_steps, total_steps):
+        self._cosine, self._base, self._min, self._warmup, self._total = True, base_lr, min_lr, warmup_steps, total_steps
+
+    def get_lr(self, step):
+        import numpy as np
+        f = np.float32
+        base, lo = f(self._base), f(self._min)
+        if self._warmup > 0 and step < self._warmup:
+            return float(base * (f(step + 1) / f(self._warmup)))
+        decay = self._total - self._warmup
+        if not self._cosine or decay <= 0:
+            return float(base)
+        prog = step - self._warmup
+        if prog >= decay:
+            return float(lo)
+        phase = f(np.pi) * f(prog) / f(decay)
+        cosine = f(0.5) * (f(1.0) + f(_libm.cosf(float(phase))))
+        return float(lo + (base - lo) * cosine)
 
 
 def _stream():
@@ -151,6 +190,78 @@ class AdamWOptimizer:
         flags = (B.CLIP_FUSED if fused_clip else 0) | (B.STEP_ZERO_GRADS if zero_grads else 0)
         self.plan.adamw(self.step_params(), flags, _stream() if stream is None else stream)
 
+    # --- optimizer state on disk (the reference's save_checkpoint is a stub, trainer.h:317-319) ----
+    CKPT_MAGIC = b"RLXOPT01"
+
+    def save_state(self, path):
+        """Writes step counter, hyper-parameters and m, v (and master) of every tensor.
+        Layout: magic, int32 step, 5 x float32 (lr, beta1, beta2, eps, weight_decay), int32 sections, then per
+        section: uint16 name length, name, uint8 dtype (1 = FP32), int64 count, uint64 sum of the data's 32-bit
+        words, data."""
+        import numpy as np
+        import torch
+        torch.cuda.synchronize()
+        st = self.store
+        secs = []
+        for i, s in enumerate(st.specs):
+            for which in ("m", "v") + (("master",) if (st.master is not None and s.dtype == DTYPE_F16) else ()):
+                secs.append((s.name + "." + which, st.state(i, which)))
+        tmp = path + ".tmp"
+        with open(tmp, "wb") as f:
+            f.write(self.CKPT_MAGIC)
+            f.write(struct.pack("<i5fi", self.step_, self.lr, self.beta1, self.beta2, self.eps, self.weight_decay,
+                                len(secs)))
+            for name, t in secs:
+                a = t.detach().cpu().numpy()
+                nb = name.encode()
+                f.write(struct.pack("<H", len(nb)) + nb)
+                f.write(struct.pack("<BqQ", 1, a.size, int(a.view(np.uint32).sum(dtype=np.uint64))))
+                f.write(a.tobytes())
+        os.replace(tmp, path)
+
+    def load_state(self, path):
+        """Restores what save_state wrote into this optimizer's store; the tensor list must be the same.
+        Raises ValueError on a foreign, truncated or corrupted file and leaves the state untouched then."""
+        import numpy as np
+        import torch
+        st = self.store
+        want = []
+        for i, s in enumerate(st.specs):
+            for which in ("m", "v") + (("master",) if (st.master is not None and s.dtype == DTYPE_F16) else ()):
+                want.append((s.name + "." + which, i, which, s.n))
+        loaded = []
+        with open(path, "rb") as f:
+            if f.read(8) != self.CKPT_MAGIC:
+                raise ValueError("not an optimizer state file: " + path)
+            head = f.read(28)
+            if len(head) != 28:
+                raise ValueError("truncated optimizer state file")
+            step, lr, b1, b2, eps, wd, nsec = struct.unpack("<i5fi", head)
+            if nsec != len(want):
+                raise ValueError("optimizer state has %d sections, this optimizer needs %d" % (nsec, len(want)))
+            for name, i, which, n in want:
+                raw = f.read(2)
+                if len(raw) != 2:
+                    raise ValueError("truncated optimizer state file")
+                (ln,) = struct.unpack("<H", raw)
+                got = f.read(ln).decode()
+                meta = f.read(17)
+                if len(meta) != 17:
+                    raise ValueError("truncated optimizer state file")
+                dt, cnt, csum = struct.unpack("<BqQ", meta)
+                if got != name or dt != 1 or cnt != n:
+                    raise ValueError("section %r (%d) does not match tensor %r (%d)" % (got, cnt, name, n))
+                a = np.frombuffer(f.read(4 * n), dtype=np.float32)
+                if a.size != n:
+                    raise ValueError("truncated optimizer state file")
+                if int(a.view(np.uint32).sum(dtype=np.uint64)) != csum:
+                    raise ValueError("checksum mismatch in section " + name)
+                loaded.append((i, which, a))
+        for i, which, a in loaded:
+            st.state(i, which).copy_(torch.from_numpy(a.copy()))
+        self.step_, self.lr, self.beta1, self.beta2, self.eps, self.weight_decay = step, lr, b1, b2, eps, wd
+        torch.cuda.synchronize()
+
     def clip_grad_norm_(self, max_norm, fused=False, stream=None):
         """Returns the pre-clip norm (blocking read, as in the reference).  fused=False scales the
         gradients in place when norm > max_norm; fused=True leaves them alone and the following
@@ -172,3 +283,96 @@ def training_step(optimizer, max_grad_norm, fused_clip=False, zero_grads=False):
         grad_norm = optimizer.clip_grad_norm_(max_grad_norm, fused=fused_clip)
     optimizer.step(fused_clip=fused_clip and clipped, zero_grads=zero_grads)
     return grad_norm
+
+
+class Logger:
+    """JSON-lines metrics logger with the reference's interface (include/training/logger.h:27-128):
+    log() accumulates, commit() writes the window's means as one object with a "step" key, appends to
+    <log_dir>/train_log.jsonl and prints a summary line.  Keys come out sorted, as the reference's
+    JSON object type orders them."""
+
+    def __init__(self, log_dir=""):
+        self._file, self._path, self._pending, self._history = None, "", {}, []
+        if log_dir:
+            self.open(log_dir)
+
+    def open(self, log_dir):
+        if not log_dir:
+            return
+        os.makedirs(log_dir, exist_ok=True)
+        self._path = os.path.join(log_dir, "train_log.jsonl")
+        self._file = open(self._path, "a")          # append: survives restarts
+
+    def log(self, step, key, value=None):
+        if isinstance(key, dict):
+            for k, v in key.items():
+                self.log(step, k, v)
+            return
+        import numpy as np
+        acc = self._pending.setdefault(key, [np.float32(0.0), 0])
+        acc[0] = np.float32(acc[0] + np.float32(value))       # FP32 accumulation, as the reference's
+        acc[1] += 1
+
+    def commit(self, step):
+        if not self._pending:
+            return
+        import numpy as np
+        obj = {"step": step}
+        parts = ["[step %d]" % step]
+        for key in sorted(self._pending):
+            total, count = self._pending[key]
+            val = float(total / np.float32(count)) if count else 0.0
+            obj[key] = val
+            parts.append(("  %s=%.3e" if (abs(val) < 0.01 and val != 0.0) else "  %s=%.4f") % (key, val))
+        print("".join(parts))
+        if self._file:
+            self._file.write(json.dumps(obj, sort_keys=True, separators=(",", ":")) + "\n")
+            self._file.flush()
+        self._history.append(obj)
+        self._pending = {}
+
+    def history(self):
+        return self._history
+
+    def last(self, key):
+        for obj in reversed(self._history):
+            if key in obj:
+                return obj[key]
+        return math.nan
+
+    def log_path(self):
+        return self._path
+
+    def close(self):
+        if self._file:
+            self._file.close()
+            self._file = None
+
+
+def train_loop(optimizer, scheduler, logger, produce_grads, total_steps, max_grad_norm=1.0, fused_clip=True,
+               logging_steps=1, save_steps=0, save_path=None, tokens_per_step=0):
+    """The optimizer end of Trainer::train (include/training/trainer.h:183-225): per step set the
+    scheduled rate, obtain gradients (produce_grads(step) stands for forward/backward and returns the
+    loss), clip, step, synchronise, log loss / lr / grad_norm / step_ms / tok_per_sec, commit every
+    logging_steps, save the optimizer state every save_steps."""
+    import torch
+    global_step = 0
+    while global_step < total_steps:
+        cur_lr = scheduler.get_lr(global_step)
+        optimizer.set_lr(cur_lr)
+        t0 = time.perf_counter()
+        loss = produce_grads(global_step)
+        grad_norm = training_step(optimizer, max_grad_norm, fused_clip=fused_clip)
+        torch.cuda.synchronize()
+        step_ms = (time.perf_counter() - t0) * 1e3
+        global_step += 1
+        logger.log(global_step, "loss", loss)
+        logger.log(global_step, "lr", cur_lr)
+        logger.log(global_step, "grad_norm", grad_norm)
+        logger.log(global_step, "step_ms", step_ms)
+        logger.log(global_step, "tok_per_sec", tokens_per_step / (step_ms * 1e-3) if step_ms > 0 else 0.0)
+        if global_step % logging_steps == 0:
+            logger.commit(global_step)
+        if save_steps > 0 and save_path and global_step % save_steps == 0:
+            optimizer.save_state(save_path)
+    return global_step

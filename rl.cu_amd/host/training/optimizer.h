@@ -10,7 +10,10 @@
 #pragma once
 #include <cassert>
 #include <cmath>
+#include <cstdint>
 #include <cstring>
+#include <string>
+#include <vector>
 
 #include "../kernels/adamw.h"
 
@@ -108,6 +111,72 @@ public:
         RLX_CHECK(rlx_plan_adamw(plan_for(grads), &sp, flags, (void*)stream));
     }
 
+    // Optimizer state on disk (the reference's save_checkpoint is a stub, trainer.h:317-319).
+    // File: "RLXOPT01", int32 step, 5 floats (lr, beta1, beta2, eps, weight_decay), int32 sections;
+    // per section: uint16 name length, name, uint8 dtype (1 = FP32), int64 count, uint64 sum of the
+    // data's 32-bit words, data.  Sections: fp16.master (if kept), fp16.m, fp16.v, fp32.m, fp32.v.
+    // Both return false (and print why) on failure; load_state leaves the state alone then.
+    bool save_state(const std::string& path) const {
+        HIP_CHECK(hipDeviceSynchronize());
+        const std::string tmp = path + ".tmp";
+        FILE* f = fopen(tmp.c_str(), "wb");
+        if (!f) { fprintf(stderr, "[AdamW] cannot write %s\n", tmp.c_str()); return false; }
+        const std::vector<Section> secs = sections();
+        const int32_t step = step_, nsec = (int32_t)secs.size();
+        const float hyper[5] = {lr, beta1, beta2, eps, weight_decay};
+        bool ok = fwrite("RLXOPT01", 1, 8, f) == 8 && fwrite(&step, 4, 1, f) == 1 && fwrite(hyper, 4, 5, f) == 5 &&
+                  fwrite(&nsec, 4, 1, f) == 1;
+        std::vector<float> host;
+        for (const Section& s : secs) {
+            host.resize(s.n);
+            HIP_CHECK(hipMemcpy(host.data(), s.dev, s.n * sizeof(float), hipMemcpyDeviceToHost));
+            const uint16_t len = (uint16_t)s.name.size();
+            const uint8_t dtype = 1;
+            const int64_t count = (int64_t)s.n;
+            const uint64_t sum = word_sum(host.data(), s.n);
+            ok = ok && fwrite(&len, 2, 1, f) == 1 && fwrite(s.name.data(), 1, len, f) == len &&
+                 fwrite(&dtype, 1, 1, f) == 1 && fwrite(&count, 8, 1, f) == 1 && fwrite(&sum, 8, 1, f) == 1 &&
+                 fwrite(host.data(), sizeof(float), s.n, f) == s.n;
+        }
+        ok = (fclose(f) == 0) && ok;
+        if (ok) ok = rename(tmp.c_str(), path.c_str()) == 0;
+        if (!ok) fprintf(stderr, "[AdamW] writing %s failed\n", path.c_str());
+        return ok;
+    }
+
+    bool load_state(const std::string& path) {
+        FILE* f = fopen(path.c_str(), "rb");
+        if (!f) { fprintf(stderr, "[AdamW] cannot read %s\n", path.c_str()); return false; }
+        const std::vector<Section> secs = sections();
+        char magic[8];
+        int32_t step = 0, nsec = 0;
+        float hyper[5];
+        bool ok = fread(magic, 1, 8, f) == 8 && memcmp(magic, "RLXOPT01", 8) == 0 && fread(&step, 4, 1, f) == 1 &&
+                  fread(hyper, 4, 5, f) == 5 && fread(&nsec, 4, 1, f) == 1 && nsec == (int32_t)secs.size();
+        std::vector<std::vector<float>> data(secs.size());
+        for (size_t i = 0; ok && i < secs.size(); i++) {
+            uint16_t len = 0;
+            uint8_t dtype = 0;
+            int64_t count = 0;
+            uint64_t sum = 0;
+            char name[256];
+            ok = fread(&len, 2, 1, f) == 1 && len < sizeof(name) && fread(name, 1, len, f) == len &&
+                 fread(&dtype, 1, 1, f) == 1 && fread(&count, 8, 1, f) == 1 && fread(&sum, 8, 1, f) == 1 &&
+                 std::string(name, len) == secs[i].name && dtype == 1 && count == (int64_t)secs[i].n;
+            if (!ok) break;
+            data[i].resize(secs[i].n);
+            ok = fread(data[i].data(), sizeof(float), secs[i].n, f) == secs[i].n &&
+                 word_sum(data[i].data(), secs[i].n) == sum;
+        }
+        fclose(f);
+        if (!ok) { fprintf(stderr, "[AdamW] %s is not a matching, intact optimizer state\n", path.c_str()); return false; }
+        for (size_t i = 0; i < secs.size(); i++)
+            HIP_CHECK(hipMemcpy(secs[i].dev, data[i].data(), secs[i].n * sizeof(float), hipMemcpyHostToDevice));
+        step_ = step;
+        lr = hyper[0]; beta1 = hyper[1]; beta2 = hyper[2]; eps = hyper[3]; weight_decay = hyper[4];
+        return true;
+    }
+
     // The multi-tensor plan over {projections, embedding, norm weights, workspace tail} for these
     // gradient pools; built on first use and rebuilt if the pools move.
     rlx_plan* plan_for(GradPools* grads) {
@@ -159,6 +228,20 @@ private:
     float* plan_float_ = nullptr;
     size_t plan_float_bytes_ = 0;
     bool embed_frozen_ = false;
+
+    struct Section { std::string name; float* dev; size_t n; };
+    std::vector<Section> sections() const {
+        std::vector<Section> s;
+        if (fp16_master_) s.push_back({"fp16.master", fp16_master_, n16_});
+        if (n16_) { s.push_back({"fp16.m", fp16_m_, n16_}); s.push_back({"fp16.v", fp16_v_, n16_}); }
+        if (n32_) { s.push_back({"fp32.m", fp32_m_, n32_}); s.push_back({"fp32.v", fp32_v_, n32_}); }
+        return s;
+    }
+    static uint64_t word_sum(const float* p, size_t n) {
+        uint64_t acc = 0;
+        for (size_t i = 0; i < n; i++) { uint32_t w; memcpy(&w, p + i, 4); acc += w; }
+        return acc;
+    }
 
     void init(const ParamPools& pools, bool use_master) {
         pools_ = pools;

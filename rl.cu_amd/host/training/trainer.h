@@ -2,6 +2,11 @@
 // and :323-352; GRPO_trainer.h:508-514 calls the same two functions): optional zeroing of the
 // embedding gradients, gradient clipping by global L2 norm, one optimizer step.
 #pragma once
+#include <chrono>
+#include <functional>
+
+#include "logger.h"
+#include "lr_scheduler.h"
 #include "optimizer.h"
 
 struct OptimStepConfig {          // the fields of TrainingConfig that this path reads (trainer.h:36-43)
@@ -55,3 +60,43 @@ private:
     OptimStepConfig config_;
     float last_grad_norm_ = 0.0f;
 };
+
+// The optimizer end of Trainer::train (include/training/trainer.h:183-225): per step set the scheduled
+// rate, obtain gradients (produce_grads(step) stands for the forward/backward passes and returns the
+// loss), clip and step, synchronise, log loss / lr / grad_norm / step_ms / tok_per_sec, commit every
+// logging_steps, save the optimizer state every save_steps.  Returns the number of steps taken.
+struct TrainLoopConfig {
+    int total_steps = 0;
+    int logging_steps = 1;
+    int save_steps = 0;               // 0: never
+    std::string save_path;            // optimizer state file
+    float tokens_per_step = 0.0f;     // global_batch_size * sequence length
+    size_t embed_elems = 0;
+};
+
+inline int run_train_loop(AdamWOptimizer& optimizer, const LRScheduler& scheduler, Logger& logger, OptimStep& tail,
+                          GradPools* grads, const std::function<float(int)>& produce_grads,
+                          const TrainLoopConfig& cfg, hipStream_t stream = 0) {
+    int global_step = 0;
+    while (global_step < cfg.total_steps) {
+        const float cur_lr = scheduler.get_lr(global_step);
+        optimizer.set_lr(cur_lr);
+        const auto t0 = std::chrono::steady_clock::now();
+        const float loss = produce_grads(global_step);
+        const float grad_norm = tail.apply(grads, cfg.embed_elems, stream);
+        HIP_CHECK(hipDeviceSynchronize());
+        const auto t1 = std::chrono::steady_clock::now();
+        const float step_ms = std::chrono::duration<float, std::milli>(t1 - t0).count();
+        const float tok_per_sec = cfg.tokens_per_step / (step_ms * 1e-3f);
+        global_step++;
+        logger.log(global_step, "loss", loss);
+        logger.log(global_step, "lr", cur_lr);
+        logger.log(global_step, "grad_norm", grad_norm);
+        logger.log(global_step, "step_ms", step_ms);
+        logger.log(global_step, "tok_per_sec", tok_per_sec);
+        if (cfg.logging_steps > 0 && global_step % cfg.logging_steps == 0) logger.commit(global_step);
+        if (cfg.save_steps > 0 && !cfg.save_path.empty() && global_step % cfg.save_steps == 0)
+            optimizer.save_state(cfg.save_path);
+    }
+    return global_step;
+}

@@ -10,10 +10,13 @@
 //   5. clip_grad_norm_ returns the pre-clip norm; clipped gradients have norm <= max; fused == unfused
 //   6. operator API (launch_adamw_fp16 / launch_adamw_fp32) on raw pointers
 //   7. frozen embedding flagged in the plan, gradients cleared inside the update
+//   8. optimizer state save / load   9. train loop with LR schedule and JSON-lines log
 // The oracle (liborc_adamw.so) is used as the checker only.
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <filesystem>
+#include <string>
 #include <vector>
 
 #include "training/trainer.h"
@@ -260,6 +263,76 @@ static void test_frozen_and_zeroing() {
     if (na == nb && diff == 0 && moved == 0 && nonzero == 0) PASS(name); else FAIL(name, "diff=%zu", diff);
 }
 
+// 8. optimizer state: save, continue, reload into a fresh optimizer, continue: identical bits
+static void test_checkpoint() {
+    const char* name = "optimizer state save / load";
+    const std::string path = "/tmp/rlx_test_opt.state";
+    Fixture a(5e-3f), b(5e-3f);
+    AdamWOptimizer oa(a.pools, 1e-3f), ob(b.pools, 1e-3f);
+    OptimStepConfig c; c.max_grad_norm = 0.25f; c.fused_clip = true;
+    OptimStep sa(&oa, c), sb(&ob, c);
+    for (int i = 0; i < 3; i++) sa.apply(&a.grads);
+    bool ok = oa.save_state(path);
+    HIP_CHECK(hipMemcpy(b.w16, a.w16, a.n16 * 2, hipMemcpyDeviceToDevice));   // weights are the model's to save
+    HIP_CHECK(hipMemcpy(b.w32, a.w32, a.n32 * 4, hipMemcpyDeviceToDevice));
+    ok = ok && ob.load_state(path) && ob.get_step() == 3;
+    for (int i = 0; i < 2; i++) { sa.apply(&a.grads); sb.apply(&b.grads); }
+    HIP_CHECK(hipDeviceSynchronize());
+    a.download(); b.download();
+    size_t diff = 0;
+    for (size_t i = 0; i < a.n16; i++) diff += a.h_w16[i] != b.h_w16[i];
+    auto ma = d2h(oa.fp16_master(), a.n16), mb = d2h(ob.fp16_master(), b.n16);
+    auto va = d2h(oa.fp32_v(), a.n32), vb = d2h(ob.fp32_v(), b.n32);
+    for (size_t i = 0; i < a.n16; i++) diff += memcmp(&ma[i], &mb[i], 4) != 0;
+    for (size_t i = 0; i < a.n32; i++) diff += memcmp(&va[i], &vb[i], 4) != 0;
+    // a damaged file is refused and changes nothing
+    FILE* f = fopen(path.c_str(), "r+b");
+    fseek(f, -9, SEEK_END); fputc(0x5A, f); fclose(f);
+    AdamWOptimizer oc(a.pools, 1e-3f);
+    bool refused = !oc.load_state(path) && oc.get_step() == 0 && !oc.load_state("/tmp/rlx_no_such_file");
+    remove(path.c_str());
+    if (ok && diff == 0 && refused && ob.get_step() == 5) PASS(name); else FAIL(name, "ok=%d diff=%zu refused=%d", ok, diff, refused);
+}
+
+// 9. scheduled learning rate, train loop, JSON-lines log
+static void test_train_loop() {
+    const char* name = "train loop with LR schedule and JSONL log";
+    const std::string dir = "/tmp/rlx_test_run";
+    std::filesystem::remove_all(dir);
+    Fixture f(5e-3f);
+    AdamWOptimizer opt(f.pools, 1e-3f);
+    LRScheduler sched;
+    sched.init_cosine(1e-3f, 1e-4f, 2, 8);
+    OptimStepConfig c; c.max_grad_norm = 0.25f; c.fused_clip = true;
+    OptimStep tail(&opt, c);
+    TrainLoopConfig lc; lc.total_steps = 8; lc.logging_steps = 2; lc.tokens_per_step = 4096.0f;
+    int steps;
+    {
+        Logger logger(dir);
+        steps = run_train_loop(opt, sched, logger, tail, &f.grads, [&](int s) {
+            RLX_CHECK(rlx_fill_f16((uint16_t*)f.g16, f.n16, 100 + s, 0, 0.0f, 5e-3f, 0, 0, 0, nullptr));
+            return 3.0f / (1 + s);
+        }, lc);
+        bool ok = steps == 8 && opt.get_step() == 8 && logger.history().size() == 4 && opt.lr == sched.get_lr(7) &&
+                  logger.history()[0].step == 2 && fabsf(logger.last("loss") - (3.0f / 7 + 3.0f / 8) / 2) < 1e-6f &&
+                  logger.last("grad_norm") > 0.25f && std::isnan(logger.last("nope"));
+        if (!ok) { FAIL(name, "loop state"); return; }
+    }
+    FILE* fp = fopen((dir + "/train_log.jsonl").c_str(), "r");
+    int lines = 0; char buf[1024]; bool shape = fp != nullptr;
+    while (fp && fgets(buf, sizeof(buf), fp)) {
+        lines++;
+        std::string l(buf);
+        shape = shape && l.rfind("{\"grad_norm\":", 0) == 0 && l.find("\"loss\":") != std::string::npos &&
+                l.find("\"lr\":") != std::string::npos && l.find("\"step\":" + std::to_string(2 * lines)) != std::string::npos &&
+                l.find("\"step_ms\":") != std::string::npos && l.find("\"tok_per_sec\":") != std::string::npos;
+    }
+    if (fp) fclose(fp);
+    std::filesystem::remove_all(dir);
+    if (shape && lines == 4 && Logger::number(1e-5) == "1e-05" && Logger::number(2.0) == "2.0") PASS(name);
+    else FAIL(name, "lines=%d shape=%d", lines, shape);
+}
+
 int main() {
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
@@ -274,6 +347,8 @@ int main() {
     test_clip();
     test_launch_api();
     test_frozen_and_zeroing();
+    test_checkpoint();
+    test_train_loop();
     printf("=== %s (%d failure%s) ===\n", g_fails ? "FAILED" : "ALL PASSED", g_fails, g_fails == 1 ? "" : "s");
     return g_fails;
 }

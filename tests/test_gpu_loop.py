@@ -1,0 +1,118 @@
+"""The callers either side of the step: scheduled learning rate, train loop with JSON-lines logging,
+optimizer-state checkpoint and resume."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+from util import bits
+
+pytestmark = pytest.mark.gpu
+
+MINI = dict(vocab=300, hidden=64, inter=128, layers=2, q_heads=4, kv_heads=2, head_dim=16, tied=True)
+
+
+def make(L, host, master):
+    specs = L.qwen3_tensor_list(MINI, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
+    st = host.ParamStore(specs, master=master)
+    st.fill("p", 1, 0.0, 0.02)
+    if master:
+        st.init_master()
+    return specs, st, host.AdamWOptimizer(st, lr=1e-3, chunk_elems=2048)
+
+
+def snapshot(st):
+    pools = [st.p16, st.p32, st.m, st.v] + ([st.master] if st.master is not None else [])
+    return [t.clone() for t in pools]
+
+
+@pytest.mark.parametrize("master", [False, True])
+def test_checkpoint_resume_is_bit_identical(L, host, torch_gpu, tmp_path, master):
+    """Three steps, save, two more steps; a fresh optimizer that loads the file and takes the same two
+    steps ends with identical bits.  Weights are the model's to save: they are copied across here."""
+    torch = torch_gpu
+    specs, st_a, opt_a = make(L, host, master)
+    for step in range(1, 4):
+        st_a.fill("g", 10 + step, 0.0, 5e-3)
+        host.training_step(opt_a, 0.5, fused_clip=True)
+    path = str(tmp_path / "opt.state")
+    opt_a.save_state(path)
+    weights = [st_a.p16.clone(), st_a.p32.clone()]
+    for step in range(4, 6):
+        st_a.fill("g", 10 + step, 0.0, 5e-3)
+        opt_a.set_lr(5e-4)
+        host.training_step(opt_a, 0.5, fused_clip=True)
+    _, st_b, opt_b = make(L, host, master)
+    st_b.p16.copy_(weights[0])
+    st_b.p32.copy_(weights[1])
+    opt_b.load_state(path)
+    assert opt_b.get_step() == 3 and abs(opt_b.lr - 1e-3) < 1e-9
+    for step in range(4, 6):
+        st_b.fill("g", 10 + step, 0.0, 5e-3)
+        opt_b.set_lr(5e-4)
+        host.training_step(opt_b, 0.5, fused_clip=True)
+    torch.cuda.synchronize()
+    assert opt_b.get_step() == 5
+    for a, b in zip(snapshot(st_a), snapshot(st_b)):
+        assert torch.equal(a, b)
+
+
+def test_checkpoint_rejects_bad_files(L, host, torch_gpu, tmp_path):
+    specs, st, opt = make(L, host, False)
+    st.fill("g", 3, 0.0, 5e-3)
+    opt.step()
+    path = str(tmp_path / "opt.state")
+    opt.save_state(path)
+    before = snapshot(st)
+    data = open(path, "rb").read()
+    cases = {"foreign": b"NOTASTATE" + data[9:], "truncated": data[: len(data) // 2],
+             "flipped": data[:-5] + bytes([data[-5] ^ 0x40]) + data[-4:]}
+    for name, blob in cases.items():
+        bad = str(tmp_path / name)
+        open(bad, "wb").write(blob)
+        with pytest.raises(ValueError):
+            opt.load_state(bad)
+        assert all(torch_gpu.equal(a, b) for a, b in zip(before, snapshot(st))), name
+    _, _, other = make(L, host, True)                      # different structure: master sections expected
+    with pytest.raises(ValueError):
+        other.load_state(path)
+
+
+def test_train_loop_logs_jsonl(L, host, torch_gpu, tmp_path, capsys):
+    """Cosine schedule with warm-up drives set_lr; every second step one JSON line with the window means of
+    loss, lr, grad_norm, step_ms, tok_per_sec (the keys of include/training/trainer.h:208-212)."""
+    specs, st, opt = make(L, host, False)
+    sched = host.LRScheduler()
+    sched.init_cosine(1e-3, 1e-4, 2, 8)
+    log_dir = str(tmp_path / "run")
+    logger = host.Logger(log_dir)
+    losses = []
+
+    def produce(step):
+        st.fill("g", 100 + step, 0.0, 5e-3)
+        losses.append(3.0 / (1 + step))
+        return losses[-1]
+
+    done = host.train_loop(opt, sched, logger, produce, total_steps=8, max_grad_norm=0.5, logging_steps=2,
+                           save_steps=4, save_path=str(tmp_path / "opt.state"), tokens_per_step=4096)
+    logger.close()
+    assert done == 8 and opt.get_step() == 8 and os.path.exists(str(tmp_path / "opt.state"))
+    rows = [json.loads(l) for l in open(os.path.join(log_dir, "train_log.jsonl"))]
+    assert [r["step"] for r in rows] == [2, 4, 6, 8]
+    assert all(sorted(r) == ["grad_norm", "loss", "lr", "step", "step_ms", "tok_per_sec"] for r in rows)
+    for k, r in enumerate(rows):
+        s0, s1 = 2 * k, 2 * k + 1
+        assert abs(r["loss"] - (losses[s0] + losses[s1]) / 2) < 1e-6
+        assert abs(r["lr"] - (sched.get_lr(s0) + sched.get_lr(s1)) / 2) < 1e-9
+        assert r["grad_norm"] > 0.5 and r["step_ms"] > 0 and r["tok_per_sec"] > 0
+    assert abs(opt.lr - sched.get_lr(7)) < 1e-12
+    assert logger.last("loss") == rows[-1]["loss"] and math.isnan(logger.last("nope")) and len(logger.history()) == 4
+    assert "[step 8]" in capsys.readouterr().out
+    # a restart appends to the same file
+    logger2 = host.Logger(log_dir)
+    logger2.log(9, {"loss": 1.0, "lr": 1e-4})
+    logger2.commit(9)
+    logger2.close()
+    assert len(open(os.path.join(log_dir, "train_log.jsonl")).readlines()) == 5
