@@ -47,7 +47,17 @@ def cpu_baseline(O, host, sample, hyper, step, seconds=8.0):
         el = time.perf_counter() - t0
         if el >= seconds or reps >= 200:
             break
+    # one thread, on the first 4 Mi parameters of the sample
+    n1 = min(p.size, 4 * 1024 * 1024)
+    one = [a[:n1].copy() for a in (p, g, m, v)]
+    O.step_fp16_threaded(None, *one, *args, 0.0, 1)
+    r1, t1 = 0, time.perf_counter()
+    while time.perf_counter() - t1 < 2.0:
+        O.step_fp16_threaded(None, *one, *args, 0.0, 1)
+        r1 += 1
+    single = n1 * r1 / (time.perf_counter() - t1)
     return {"value": p.size * reps / el, "unit": "params/s", "cores": threads, "kind": "port",
+            "single_thread_value": single,
             "sample": "%d-parameter slice of embed_tokens (p, g, m, v after 99 steps), %d repeated steps, "
                       "%.1f s wall; oracle's threaded AdamW loop, gcc -O3, no FMA contraction" % (p.size, reps, el),
             "gbps": BYTES_UPDATE * p.size * reps / el / 1e9}
