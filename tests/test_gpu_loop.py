@@ -116,3 +116,31 @@ def test_train_loop_logs_jsonl(L, host, torch_gpu, tmp_path, capsys):
     logger2.commit(9)
     logger2.close()
     assert len(open(os.path.join(log_dir, "train_log.jsonl")).readlines()) == 5
+
+
+def test_steps_reduce_a_loss(L, host, torch_gpu):
+    """The last case of the reference's own test (tests/test_adamw.cu:453-501: five steps at lr=1e-4 reduce
+    the model's NLL), on a loss that needs no model: 0.5 * |p - target|^2 with its exact gradient."""
+    torch = torch_gpu
+    specs = [L.TensorSpec("w", 50_000, L.DTYPE_F16, 0, 0), L.TensorSpec("n", 500, L.DTYPE_F32, L.NO_DECAY, 0)]
+    st = host.ParamStore(specs, master=True)
+    st.fill("p", 1, 0.0, 0.5)
+    st.init_master()
+    target16 = torch.full((50_000,), 0.25, dtype=torch.float16, device="cuda:0")
+    target32 = torch.full((500,), -0.5, dtype=torch.float32, device="cuda:0")
+    opt = host.AdamWOptimizer(st, lr=1e-2, weight_decay=0.0)
+
+    def loss_and_grads():
+        d16 = st.param(0).float() - target16.float()
+        d32 = st.param(1) - target32
+        st.grad(0).copy_(d16.half())
+        st.grad(1).copy_(d32)
+        return 0.5 * (d16.pow(2).sum() + d32.pow(2).sum()).item()
+
+    losses = []
+    for _ in range(5):
+        losses.append(loss_and_grads())
+        host.training_step(opt, 1.0, fused_clip=True)
+    losses.append(loss_and_grads())
+    assert all(b < a for a, b in zip(losses, losses[1:])), losses
+    assert opt.get_step() == 5
