@@ -66,12 +66,18 @@ _lib = None
 
 
 def load():
-    """Loads the built library; raises if it has not been built (no fallback of any kind)."""
+    """Loads the built library, compiling it first if it is missing; raises if that fails (there is no
+    CPU fallback of any kind)."""
     global _lib
     if _lib is not None:
         return _lib
     if not os.path.exists(LIB_PATH):
-        raise RuntimeError("librlx_adamw.so is not built (%s); run __graft_entry__.build()" % LIB_PATH)
+        # nothing built yet: compile now (hipcc); if that fails there is nothing to fall back to
+        from . import build as _build
+        try:
+            _build.build_library()
+        except Exception as exc:
+            raise RuntimeError("librlx_adamw.so is not built (%s) and building it failed: %s" % (LIB_PATH, exc))
     try:
         # torch, when present, brings its own HIP runtime: load it first so that this library
         # binds to the same runtime instance as the tensors it is handed.
