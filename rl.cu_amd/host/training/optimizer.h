@@ -36,6 +36,30 @@ struct ParamPools {
     size_t proj_elems = 0;
     float* fp32_pool = nullptr;
     size_t fp32_pool_elems = 0;
+    // Optional per-layer structure, only used by the (layer, tensor) accessors below:
+    // sizes of q, k, v, o, gate, up, down and of input_norm, q_norm, k_norm, post_attn_norm.
+    int num_layers = 0;
+    size_t proj_sizes[7] = {};
+    size_t norm_sizes[4] = {};
+
+    // Fills sizes and structure from the model dimensions (include/model/config.h:5-30; pool order
+    // of include/training/optimizer.h:30-32).  The pool pointers stay for the caller to set.
+    static ParamPools for_qwen3(int num_layers, int hidden, int q_dim, int kv_dim, int intermediate, int head_dim,
+                                int vocab) {
+        ParamPools p;
+        const size_t H = (size_t)hidden;
+        const size_t ps[7] = {(size_t)q_dim * H, (size_t)kv_dim * H, (size_t)kv_dim * H, H * (size_t)q_dim,
+                              (size_t)intermediate * H, (size_t)intermediate * H, H * (size_t)intermediate};
+        const size_t ns[4] = {H, (size_t)head_dim, (size_t)head_dim, H};
+        size_t per16 = 0, per32 = 0;
+        for (int i = 0; i < 7; i++) { p.proj_sizes[i] = ps[i]; per16 += ps[i]; }
+        for (int i = 0; i < 4; i++) { p.norm_sizes[i] = ns[i]; per32 += ns[i]; }
+        p.num_layers = num_layers;
+        p.proj_elems = per16 * (size_t)num_layers;
+        p.fp16_pool_elems = p.proj_elems + (size_t)vocab * H;
+        p.fp32_pool_elems = per32 * (size_t)num_layers + H;
+        return p;
+    }
 };
 
 // The gradient pools (Qwen3Gradients, include/model/qwen3.h:190-218).  float_pool may be longer
@@ -87,6 +111,17 @@ public:
     float* fp32_v() { return fp32_v_; }
     size_t num_fp16_params() const { return n16_; }
     size_t num_fp32_params() const { return n32_; }
+
+    // Test accessors by (layer, tensor), as in the reference (optimizer.h:107-116); they need the
+    // per-layer structure in ParamPools.  proj: 0=q 1=k 2=v 3=o 4=gate 5=up 6=down;
+    // norm: 0=input 1=q 2=k 3=post_attn.
+    float* get_fp16_master(int layer, int proj) const { return fp16_master_ ? fp16_master_ + fp16_offset(layer, proj) : nullptr; }
+    float* get_fp16_m(int layer, int proj) const { return fp16_m_ + fp16_offset(layer, proj); }
+    float* get_fp16_v(int layer, int proj) const { return fp16_v_ + fp16_offset(layer, proj); }
+    float* get_fp32_m_norm(int layer, int norm) const { return fp32_m_ + fp32_offset(layer, norm); }
+    float* get_fp32_v_norm(int layer, int norm) const { return fp32_v_ + fp32_offset(layer, norm); }
+    float* get_final_norm_m() const { return fp32_m_ + fp32_offset(pools_.num_layers, 0); }
+    float* get_final_norm_v() const { return fp32_v_ + fp32_offset(pools_.num_layers, 0); }
 
     // Treat the embedding (the tail of the FP16 pool) as frozen: its gradients count as zero in the
     // norm and the update leaves it alone, instead of clearing the gradients and streaming an
@@ -228,6 +263,19 @@ private:
     float* plan_float_ = nullptr;
     size_t plan_float_bytes_ = 0;
     bool embed_frozen_ = false;
+
+    size_t fp16_offset(int layer, int proj) const {
+        assert(pools_.num_layers > 0 && layer >= 0 && layer < pools_.num_layers && proj >= 0 && proj < 7);
+        size_t per = 0, off = 0;
+        for (int i = 0; i < 7; i++) { per += pools_.proj_sizes[i]; if (i < proj) off += pools_.proj_sizes[i]; }
+        return (size_t)layer * per + off;
+    }
+    size_t fp32_offset(int layer, int norm) const {
+        assert(pools_.num_layers > 0 && layer >= 0 && layer <= pools_.num_layers && norm >= 0 && norm < 4);
+        size_t per = 0, off = 0;
+        for (int i = 0; i < 4; i++) { per += pools_.norm_sizes[i]; if (i < norm) off += pools_.norm_sizes[i]; }
+        return (size_t)layer * per + off;
+    }
 
     struct Section { std::string name; float* dev; size_t n; };
     std::vector<Section> sections() const {

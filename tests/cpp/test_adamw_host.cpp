@@ -171,6 +171,21 @@ static void test_step_counter() {
     for (int i = 0; i < 3; i++) opt.step(&f.grads);
     HIP_CHECK(hipDeviceSynchronize());
     ok = ok && opt.get_step() == 3;
+    // (layer, tensor) accessors follow the pool order of the reference
+    ParamPools q = ParamPools::for_qwen3(28, 1024, 2048, 1024, 3072, 128, 151936);
+    ok = ok && q.fp16_pool_elems == 595984384u && q.fp32_pool_elems == 65536u && q.proj_elems == 440401920u;
+    ParamPools small = ParamPools::for_qwen3(2, 32, 64, 16, 80, 16, 1000);
+    ok = ok && small.fp16_pool_elems == f.n16 && small.proj_elems == f.proj_n && small.fp32_pool_elems == 224u;
+    small.fp16_pool = f.w16; small.fp32_pool = f.w32;
+    {
+        AdamWOptimizer lay(small, 1e-4f);
+        const size_t per16 = 12800, q = 64 * 32, kv = 16 * 32;
+        ok = ok && lay.get_fp16_m(0, 0) == lay.fp16_m() && lay.get_fp16_m(1, 0) == lay.fp16_m() + per16 &&
+             lay.get_fp16_v(0, 3) == lay.fp16_v() + q + 2 * kv &&
+             lay.get_fp16_master(1, 6) == lay.fp16_master() + 2 * per16 - 32 * 80 &&
+             lay.get_fp32_m_norm(1, 2) == lay.fp32_m() + 96 + 32 + 16 &&
+             lay.get_final_norm_v() == lay.fp32_v() + 192;
+    }
     AdamWOptimizer moved(std::move(opt));
     ok = ok && moved.get_step() == 3 && opt.fp16_m() == nullptr;
     moved.set_lr(5e-5f);
