@@ -4,10 +4,7 @@ import json
 import math
 import os
 
-import numpy as np
 import pytest
-
-from util import bits
 
 pytestmark = pytest.mark.gpu
 

@@ -318,7 +318,6 @@ def test_device_resident_step_params_and_graph_replay(O, L, host, B, torch_gpu):
     """norm + fused-clip update recorded once as a HIP graph and replayed for several steps; between
     replays the host rewrites the 28 bytes of hyper-parameters on the device and new gradients arrive.
     Every replay is checked against the oracle, with eager work and synchronisations in between."""
-    import ctypes as C
     torch = torch_gpu
     specs = L.qwen3_tensor_list(MINI, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
     st = host.ParamStore(specs)
@@ -341,9 +340,6 @@ def test_device_resident_step_params_and_graph_replay(O, L, host, B, torch_gpu):
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.stream(side):
-        # warm-up launch outside capture, on a throw-away copy of nothing: the kernels need no lazy init,
-        # but torch wants the capture stream used once
-        torch.cuda.synchronize()
         with torch.cuda.graph(graph, stream=side):
             s = torch.cuda.current_stream().cuda_stream
             opt.plan.grad_norm(0.5, s)
@@ -366,7 +362,6 @@ def test_device_resident_step_params_and_graph_replay(O, L, host, B, torch_gpu):
         assert sum_sq == O.sumsq_mirror([h["g"] for h in hs], 2048)[0]
         oracle_step(O, L, specs, hs, step, dict(HYPER, lr=lr), clip_scale=scale)
         assert compare(st, hs, "replay %d" % step) == 0
-    del C
 
 
 def test_clip_rounds_twice_for_every_half_and_many_scales(O, L, host, B, torch_gpu):
