@@ -168,3 +168,35 @@ def test_qwen3_8b_resident(O, L, host, torch_gpu):
     # a second, identical run of the norm gives the same bits
     opt.plan.grad_norm(1.0)
     assert opt.plan.norm_read() == (n2, scale, sum_sq)
+
+
+def test_single_tensor_beyond_int32(O, B, host, torch_gpu):
+    """One flat tensor of 2^31 + 1001 parameters through the operator API (the reference's `int n` cannot
+    express it): several launches, byte offsets beyond 2^32, an odd tail.  Slices at the start, across the
+    2^31 boundary and at the very end are replayed by the oracle."""
+    torch = torch_gpu
+    n = 2 ** 31 + 1001
+    free, _ = torch.cuda.mem_get_info()
+    if free < 30 * 2 ** 30:
+        pytest.skip("needs 30 GB of free device memory")
+    p = torch.empty(n, dtype=torch.float16, device="cuda:0")
+    g = torch.empty(n, dtype=torch.float16, device="cuda:0")
+    m = torch.empty(n, dtype=torch.float32, device="cuda:0")
+    v = torch.empty(n, dtype=torch.float32, device="cuda:0")
+    B.fill_f16(p.data_ptr(), n, 1, 0.0, 0.02)
+    B.fill_f16(g.data_ptr(), n, 2, 0.0, 1e-3)
+    B.fill_f32(m.data_ptr(), n, 3, 0.0, 1e-4)
+    B.fill_f32(v.data_ptr(), n, 4, 1e-8, 1e-8, flags=1)
+    torch.cuda.synchronize()
+    slices = [(0, 3000), (2 ** 31 - 1500, 2400), (n - 1001 - 300, 1301), (123456789 * 8 + 3, 2000)]
+    ref = [dict(p=bits(p[lo: lo + k]), g=bits(g[lo: lo + k]), m=bits(m[lo: lo + k]), v=bits(v[lo: lo + k]))
+           for lo, k in slices]
+    assert np.array_equal(ref[1]["g"], O.fill_f16(2400, 2, 0.0, 1e-3, first=2 ** 31 - 1500))
+    bc1, bc2 = host.bias_correction(0.9, 7), host.bias_correction(0.999, 7)
+    assert B.adamw_fp16(None, p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), n, 1e-4, 0.9, 0.999, 1e-8,
+                        0.01, bc1, bc2) == B.OK
+    torch.cuda.synchronize()
+    for (lo, k), r in zip(slices, ref):
+        O.adamw_fp16(None, r["p"], r["g"], r["m"], r["v"], 1e-4, 0.9, 0.999, 1e-8, 0.01, bc1, bc2)
+        assert np.array_equal(bits(p[lo: lo + k]), r["p"]), lo
+        assert np.array_equal(bits(m[lo: lo + k]), r["m"]) and np.array_equal(bits(v[lo: lo + k]), r["v"]), lo
