@@ -792,6 +792,7 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
     }
     if (e != hipSuccess) {
         int st = hip_fail(e, "rlx_plan_create");
+        if (e == hipErrorNoDevice || e == hipErrorInvalidDevice) st = RLX_ERR_NO_DEVICE;
         rlx_plan_destroy(p);
         return st;
     }

@@ -127,3 +127,19 @@ def test_host_bias_correction_matches_oracle(host, O):
     for beta in (0.9, 0.999, 0.5):
         for t in (1, 2, 99, 100, 1000):
             assert host.bias_correction(beta, t) == O.bias_correction(beta, t)
+
+
+def test_plan_create_without_a_device_reports_an_error(B):
+    """Valid descriptors on a machine without a GPU: a status and a message, no crash.  (On a machine with
+    a GPU the plan is only a table of addresses: it is created and destroyed without touching them.)"""
+    lib = B.load()
+    h = C.c_void_p()
+    d = B.TensorDesc(0x10000, 0x20000, 0x30000, 0x40000, None, 5000, B.DTYPE_F16, 0)
+    st = lib.rlx_plan_create((B.TensorDesc * 1)(d), 1, 0, C.byref(h))
+    if st == B.OK:
+        assert lib.rlx_plan_num_chunks(h) == 3 and lib.rlx_plan_num_elements(h) == 5000
+        assert lib.rlx_plan_chunk_elems(h) == 2048
+        assert lib.rlx_plan_destroy(h) == B.OK
+    else:
+        assert st in (B.ERR_HIP, B.ERR_NO_DEVICE) and h.value is None
+        assert lib.rlx_last_hip_error() != b""
