@@ -401,3 +401,58 @@ def test_clip_rounds_twice_for_every_half_and_many_scales(O, L, host, B, torch_g
             once = (O.h2f(vals).astype(np.float64) * np.float64(np.float32(scale))).astype(np.float16).view(np.uint16)
         mismatches_if_fused += int((once != want).sum())
     assert mismatches_if_fused >= 3, "the scales chosen would not have told one rounding from two"
+
+
+def test_element_by_element_paths_with_master_fp32_and_half_precision_workspace(O, L, host, B, torch_gpu):
+    """Less travelled combinations in one plan: an FP16 tensor with a master copy that starts at an odd
+    element (element-by-element path), an FP32 tensor aligned to 4 but not 8 bytes, an FP16 grad-only
+    buffer; norm, fused clip, gradient clearing."""
+    torch = torch_gpu
+    n16, n32, nw = 5003, 1001, 300
+    p = torch.empty(n16 + 8, dtype=torch.float16, device="cuda:0")
+    g = torch.empty(n16 + 8, dtype=torch.float16, device="cuda:0")
+    m = torch.zeros(n16 + 8, dtype=torch.float32, device="cuda:0")
+    v = torch.zeros(n16 + 8, dtype=torch.float32, device="cuda:0")
+    w = torch.empty(n16 + 8, dtype=torch.float32, device="cuda:0")
+    p32 = torch.empty(n32 + 8, dtype=torch.float32, device="cuda:0")
+    g32 = torch.empty(n32 + 8, dtype=torch.float32, device="cuda:0")
+    m32 = torch.zeros(n32 + 8, dtype=torch.float32, device="cuda:0")
+    v32 = torch.zeros(n32 + 8, dtype=torch.float32, device="cuda:0")
+    ws = torch.empty(nw + 8, dtype=torch.float16, device="cuda:0")
+    B.fill_f16(p.data_ptr(), n16 + 8, 1, 0.0, 0.02)
+    B.fill_f16(g.data_ptr(), n16 + 8, 2, 0.0, 5e-3)
+    B.fill_f32(p32.data_ptr(), n32 + 8, 3, 1.0, 0.05)
+    B.fill_f32(g32.data_ptr(), n32 + 8, 4, 0.0, 5e-3)
+    B.fill_f16(ws.data_ptr(), nw + 8, 5, 0.0, 0.05)
+    B.check(B.fp16_to_fp32(w.data_ptr(), p.data_ptr(), n16 + 8), "fp16_to_fp32")
+    torch.cuda.synchronize()
+    o16, o32, ow = 1, 1, 3
+    descs = [B.TensorDesc(p.data_ptr() + 2 * o16, g.data_ptr() + 2 * o16, m.data_ptr() + 4 * o16,
+                          v.data_ptr() + 4 * o16, w.data_ptr() + 4 * o16, n16, B.DTYPE_F16, 0),
+             B.TensorDesc(p32.data_ptr() + 4 * o32, g32.data_ptr() + 4 * o32, m32.data_ptr() + 4 * o32,
+                          v32.data_ptr() + 4 * o32, None, n32, B.DTYPE_F32, B.TENSOR_NO_DECAY),
+             B.TensorDesc(None, ws.data_ptr() + 2 * ow, None, None, None, nw, B.DTYPE_F16, B.TENSOR_GRAD_ONLY)]
+    hp, hg, hw = bits(p), bits(g), bits(w)
+    hm, hv = np.zeros(n16 + 8, np.float32), np.zeros(n16 + 8, np.float32)
+    hp32, hg32 = bits(p32), bits(g32)
+    hm32, hv32 = np.zeros(n32 + 8, np.float32), np.zeros(n32 + 8, np.float32)
+    hws = bits(ws)
+    s16, s32, sw = slice(o16, o16 + n16), slice(o32, o32 + n32), slice(ow, ow + nw)
+    plan = B.Plan(descs, 2048)
+    plan.grad_norm(0.1)
+    norm, scale, sum_sq = plan.norm_read()
+    assert sum_sq == O.sumsq_mirror([hg[s16], hg32[s32], hws[sw]], 2048)[0] and norm > 0.1
+    sp = B.StepParams(1e-3, 0.9, 0.999, 1e-8, 0.01, host.bias_correction(0.9, 1), host.bias_correction(0.999, 1))
+    plan.adamw(sp, B.CLIP_FUSED | B.STEP_ZERO_GRADS)
+    torch.cuda.synchronize()
+    O.adamw_fp16(hw[s16], hp[s16], hg[s16], hm[s16], hv[s16], 1e-3, 0.9, 0.999, 1e-8, 0.01, sp.bias_correction1,
+                 sp.bias_correction2, clip_scale=scale)
+    O.adamw_fp32(hp32[s32], hg32[s32], hm32[s32], hv32[s32], 1e-3, 0.9, 0.999, 1e-8, 0.0, sp.bias_correction1,
+                 sp.bias_correction2, clip_scale=scale)
+    hg[s16] = 0
+    hg32[s32] = 0
+    hws[sw] = 0
+    for got, want in ((p, hp), (g, hg), (m, hm), (v, hv), (w, hw), (p32, hp32), (g32, hg32), (m32, hm32), (v32, hv32),
+                      (ws, hws)):
+        assert np.array_equal(bits(got), want)              # inside as the oracle says, outside untouched
+    plan.destroy()
