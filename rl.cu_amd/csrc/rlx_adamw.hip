@@ -270,12 +270,12 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         // no update here; the buffer is only cleared for the next accumulation
         if (zero_grads) {
             if (vec) {
-                if (is_f32) stg<true>((FV*)((float*)r.g + i0), FV{});
-                else stg<true>((HV*)((uint16_t*)r.g + i0), HV{});
+                if (is_f32) st_stream<SP>((FV*)((float*)r.g + i0), FV{});
+                else st_stream<SP>((HV*)((uint16_t*)r.g + i0), HV{});
             } else {
                 for (int e = e0; e < e0 + E && e < n_here; e++) {
-                    if (is_f32) stg<true>((float*)r.g + off + e, 0.0f);
-                    else stg<true>((uint16_t*)r.g + off + e, (uint16_t)0);
+                    if (is_f32) st_stream<SP>((float*)r.g + off + e, 0.0f);
+                    else st_stream<SP>((uint16_t*)r.g + off + e, (uint16_t)0);
                 }
             }
         }
@@ -296,10 +296,10 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         for (int e = e0; e < e0 + E && e < n_here; e++) {
             if (is_f32) {
                 update_scalar32(r, off + e, h, wd, scale, clip);
-                if (zero_grads) stg<true>((float*)r.g + off + e, 0.0f);
+                if (zero_grads) st_stream<SP>((float*)r.g + off + e, 0.0f);
             } else {
                 update_scalar16(r, off + e, h, wd, scale, clip);
-                if (zero_grads) stg<true>((uint16_t*)r.g + off + e, (uint16_t)0);
+                if (zero_grads) st_stream<SP>((uint16_t*)r.g + off + e, (uint16_t)0);
             }
         }
         return;
@@ -326,7 +326,7 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         st_stream<SP>((FV*)(r.v + i0), pack_f<E>(v));
         if (has_master) st_stream<SP>((FV*)(r.master + i0), pack_f<E>(w));
         st_stream<SP>((HV*)((uint16_t*)r.p + i0), pack_h<E>(w));
-        if (zero_grads) stg<true>((HV*)((uint16_t*)r.g + i0), HV{});
+        if (zero_grads) st_stream<SP>((HV*)((uint16_t*)r.g + i0), HV{});
     } else {
         // FP32 parameters (norm weights): the same update, in place (adamw.cu:80-90)
         unpack_f<E>(ldg<true>((const FV*)((const float*)r.g + i0)), g);
@@ -342,7 +342,7 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         st_stream<SP>((FV*)(r.m + i0), pack_f<E>(m));
         st_stream<SP>((FV*)(r.v + i0), pack_f<E>(v));
         st_stream<SP>((FV*)((float*)r.p + i0), pack_f<E>(w));
-        if (zero_grads) stg<true>((FV*)((float*)r.g + i0), FV{});
+        if (zero_grads) st_stream<SP>((FV*)((float*)r.g + i0), FV{});
     }
 }
 
@@ -496,7 +496,7 @@ __global__ __launch_bounds__(kNormBlock) void scale_grads_kernel(
 #pragma unroll
                     for (int k = 0; k < 4; k++)
                         x[k] = scaled_f16_bits(h2f(x[k] & 0xFFFFu), scale) | (scaled_f16_bits(h2f(x[k] >> 16), scale) << 16);
-                    stg<true>((u32x4*)(g + off), x);
+                    st_stream<1>((u32x4*)(g + off), x);
                 } else {
                     for (int64_t i = off; i < off + kVec && i < count; i++)
                         g[i] = (uint16_t)scaled_f16_bits(h2f(g[i]), scale);
