@@ -456,3 +456,96 @@ def test_element_by_element_paths_with_master_fp32_and_half_precision_workspace(
                       (ws, hws)):
         assert np.array_equal(bits(got), want)              # inside as the oracle says, outside untouched
     plan.destroy()
+
+
+@pytest.mark.parametrize("seed", list(range(12)))
+def test_random_plans(O, L, host, B, torch_gpu, seed):
+    """Seeded random tensor lists: sizes from 1 to 70,000, both dtypes, any start alignment, master copy or
+    not, no-decay / frozen / grad-only flags, every chunk size, two steps with norm, fused or unfused clip
+    and optional gradient clearing; every byte of every buffer (guard zones included) against the oracle."""
+    torch = torch_gpu
+    rng = np.random.default_rng(1000 + seed)
+    count = int(rng.integers(1, 14))
+    chunk = int(rng.choice([2048, 4096, 8192, 32768]))
+    fused = bool(rng.integers(0, 2))
+    zero = bool(rng.integers(0, 2))
+    max_norm = float(rng.choice([0.0, 0.05, 1e6]))
+    tensors, descs = [], []
+    for t in range(count):
+        n = int(rng.choice([rng.integers(1, 40), rng.integers(40, 3000), rng.integers(3000, 70000)]))
+        f32 = bool(rng.integers(0, 4) == 0)
+        flags = int(rng.choice([0, 0, B.TENSOR_NO_DECAY, B.TENSOR_FROZEN | B.TENSOR_NO_DECAY, B.TENSOR_GRAD_ONLY]))
+        master = (not f32) and bool(rng.integers(0, 3) == 0) and not (flags & B.TENSOR_GRAD_ONLY)
+        off = int(rng.integers(0, 9))
+        tot = n + 16
+        dt = torch.float32 if f32 else torch.float16
+        es = 4 if f32 else 2
+        d = dict(n=n, f32=f32, flags=flags, off=off, master=master)
+        d["p"] = torch.empty(tot, dtype=dt, device="cuda:0")
+        d["g"] = torch.empty(tot, dtype=dt, device="cuda:0")
+        (B.fill_f32 if f32 else B.fill_f16)(d["p"].data_ptr(), tot, 10 * t + 1, 0.0, 0.02)
+        (B.fill_f32 if f32 else B.fill_f16)(d["g"].data_ptr(), tot, 10 * t + 2, 0.0, 5e-3)
+        d["m"] = torch.empty(tot, dtype=torch.float32, device="cuda:0")
+        d["v"] = torch.empty(tot, dtype=torch.float32, device="cuda:0")
+        frozen = bool(flags & B.TENSOR_FROZEN)
+        B.fill_f32(d["m"].data_ptr(), tot, 10 * t + 3, 0.0, 0.0 if frozen else 1e-4)
+        B.fill_f32(d["v"].data_ptr(), tot, 10 * t + 4, 0.0 if frozen else 1e-8, 0.0 if frozen else 1e-8, flags=1)
+        d["w"] = torch.empty(tot, dtype=torch.float32, device="cuda:0") if master else None
+        if master:
+            B.check(B.fp16_to_fp32(d["w"].data_ptr(), d["p"].data_ptr(), tot), "fp16_to_fp32")
+        grad_only = bool(flags & B.TENSOR_GRAD_ONLY)
+        descs.append(B.TensorDesc(None if grad_only else d["p"].data_ptr() + es * off, d["g"].data_ptr() + es * off,
+                                  None if grad_only else d["m"].data_ptr() + 4 * off,
+                                  None if grad_only else d["v"].data_ptr() + 4 * off,
+                                  d["w"].data_ptr() + 4 * off if master else None, n,
+                                  B.DTYPE_F32 if f32 else B.DTYPE_F16, flags))
+        tensors.append(d)
+    torch.cuda.synchronize()
+    host_side = [{k: bits(d[k]) for k in ("p", "g", "m", "v", "w") if d[k] is not None} for d in tensors]
+    plan = B.Plan(descs, chunk)
+    for step in (1, 2):
+        scale = None
+        if max_norm > 0:
+            plan.grad_norm(max_norm)
+            norm, scale, sum_sq = plan.norm_read()
+            # frozen tensors contribute zero partials in their place of the fixed order
+            mirror, parts = O.sumsq_mirror([h["g"][d["off"]: d["off"] + d["n"]] if not d["flags"] & B.TENSOR_FROZEN
+                                            else np.zeros(d["n"], h["g"].dtype) for d, h in zip(tensors, host_side)],
+                                           chunk)
+            assert sum_sq == mirror and parts.size == plan.num_chunks
+            assert scale == O.clip_scale(np.float32(sum_sq), max_norm)[0]
+            if not fused:
+                plan.scale_grads()
+                for d, h in zip(tensors, host_side):
+                    if d["flags"] & B.TENSOR_FROZEN or scale == 1.0:
+                        continue
+                    sl = slice(d["off"], d["off"] + d["n"])
+                    (O.scale_float if d["f32"] else O.scale_half)(h["g"][sl], scale)
+        bc1, bc2 = host.bias_correction(0.9, step), host.bias_correction(0.999, step)
+        sp = B.StepParams(1e-3, 0.9, 0.999, 1e-8, 0.01, bc1, bc2)
+        use_fused = fused and max_norm > 0
+        plan.adamw(sp, (B.CLIP_FUSED if use_fused else 0) | (B.STEP_ZERO_GRADS if zero else 0))
+        torch.cuda.synchronize()
+        for d, h in zip(tensors, host_side):
+            sl = slice(d["off"], d["off"] + d["n"])
+            skip = d["flags"] & (B.TENSOR_FROZEN | B.TENSOR_GRAD_ONLY)
+            if not skip:
+                wd = 0.0 if d["flags"] & B.TENSOR_NO_DECAY else 0.01
+                cs = scale if use_fused else None
+                if d["f32"]:
+                    O.adamw_fp32(h["p"][sl], h["g"][sl], h["m"][sl], h["v"][sl], 1e-3, 0.9, 0.999, 1e-8, wd, bc1, bc2,
+                                 clip_scale=cs)
+                else:
+                    O.adamw_fp16(h["w"][sl] if d["master"] else None, h["p"][sl], h["g"][sl], h["m"][sl], h["v"][sl],
+                                 1e-3, 0.9, 0.999, 1e-8, wd, bc1, bc2, clip_scale=cs)
+            if zero:
+                h["g"][sl] = 0
+            for k in h:
+                assert np.array_equal(bits(d[k]), h[k]), "seed %d step %d tensor %s buffer %s" % (seed, step, d, k)
+        # fresh gradients for the second step
+        for t, (d, h) in enumerate(zip(tensors, host_side)):
+            (B.fill_f32 if d["f32"] else B.fill_f16)(d["g"].data_ptr(), d["n"] + 16, 100 + 10 * t + step, 0.0, 5e-3)
+        torch.cuda.synchronize()
+        for d, h in zip(tensors, host_side):
+            h["g"] = bits(d["g"])
+    plan.destroy()
