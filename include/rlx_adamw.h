@@ -172,7 +172,8 @@ int rlx_plan_adamw_dev(rlx_plan* plan, const rlx_step_params* dev_params, int st
 
 /* ------------------------------------------------------------------------------------
  * Launch tuning (process-wide; for measurement).  Unknown keys return RLX_ERR_INVALID_ARG.
- *   "update_variant"  0..N-1   which compiled tile shape of the update kernel (0 = default)
+ *   "update_variant"  0..N-1   which compiled form of the update kernel: tile shape, XCD swizzle,
+ *                              store policy (0 = default)
  *   "norm_grid"       0 = one workgroup per chunk, >0 = that many persistent workgroups
  *   "norm_nt"         1 = non-temporal loads in the norm pass (default), 0 = plain
  * ---------------------------------------------------------------------------------- */
