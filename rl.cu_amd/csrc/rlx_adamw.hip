@@ -18,7 +18,7 @@
 // grid-stride loops do not.  Consecutive workgroups go round-robin to the 8 XCDs; an optional
 // swizzle (K > 1) hands each XCD K neighbouring tiles, which did not pay in measurements.
 //
-// Norm kernel: one workgroup of 256 lanes per chunk with 128-bit reads; one FP64 partial
+// Norm kernel: one workgroup of 512 lanes per chunk with 128-bit reads; one FP64 partial
 // per chunk in a fixed slot, then a single-workgroup pass in fixed order (no atomics).
 //
 // Arithmetic follows src/kernels/adamw.cu:25-39 of the reference operation by operation
@@ -38,9 +38,11 @@
 
 namespace {
 
-constexpr int kNormBlock = 256;               // lanes per workgroup of the norm and scale passes
-constexpr int kVec = 8;                       // elements per lane per group there
-constexpr int kGroup = kNormBlock * kVec;     // 2048
+constexpr int kVec = 8;                       // elements per lane per group in the norm and scale passes
+constexpr int kNormBlock = 512;               // lanes per workgroup of the norm pass (8 wavefronts)
+constexpr int kNormGroup = kNormBlock * kVec; // 4096
+constexpr int kScaleBlock = 256;              // lanes per workgroup of the scale pass
+constexpr int kGroup = kScaleBlock * kVec;    // 2048
 constexpr int64_t kMinChunk = 2048;
 constexpr int64_t kBigChunk = 8192;
 constexpr int kFinalBlock = 1024;
@@ -348,10 +350,11 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
 
 // ---------------------------------------------------------------------------------------
 // Norm pass 1: one workgroup per chunk, one FP64 partial per chunk in the chunk's own slot.
-// Order inside a chunk (restated on the CPU by the test oracle): lane t adds x*x of its
-// 8-element groups t, t+256, ... element by element into one FP32 accumulator; the 64
-// lanes of a wavefront combine by xor butterfly with masks 32,16,8,4,2,1; the four
-// wavefront sums go through LDS and are added in FP64 in wavefront order.
+// Order inside a chunk (restated on the CPU by the test oracle): lane t of 512 adds x*x of its
+// 8-element groups t, t+512, ... element by element into one FP32 accumulator; the 64
+// lanes of a wavefront combine by xor butterfly with masks 32,16,8,4,2,1; the eight
+// wavefront sums go through LDS and are added in FP64 in wavefront order.  (512 lanes with
+// two 128-bit reads each measured 7.3 TB/s as a stand-alone stream, 256 lanes with four 6.95.)
 // ---------------------------------------------------------------------------------------
 
 template <bool NT>
@@ -373,13 +376,13 @@ __global__ __launch_bounds__(kNormBlock) void sumsq_partials_kernel(
             const uint16_t* g = (const uint16_t*)r.g;
             int64_t done = 0;
             if (aligned) {
-                for (; done + 4 * (int64_t)kGroup <= count; done += 4 * (int64_t)kGroup) {
-                    u32x4 x[4];
+                for (; done + 2 * (int64_t)kNormGroup <= count; done += 2 * (int64_t)kNormGroup) {
+                    u32x4 x[2];
 #pragma unroll
-                    for (int j = 0; j < 4; j++)
+                    for (int j = 0; j < 2; j++)
                         x[j] = ldg<NT>((const u32x4*)(g + done + (int64_t)(j * kNormBlock + tid) * kVec));
 #pragma unroll
-                    for (int j = 0; j < 4; j++) {
+                    for (int j = 0; j < 2; j++) {
 #pragma unroll
                         for (int k = 0; k < 4; k++) {
                             float a = h2f(x[j][k] & 0xFFFFu), b = h2f(x[j][k] >> 16);
@@ -389,7 +392,7 @@ __global__ __launch_bounds__(kNormBlock) void sumsq_partials_kernel(
                     }
                 }
             }
-            for (; done < count; done += kGroup) {
+            for (; done < count; done += kNormGroup) {
                 const int64_t off = done + (int64_t)tid * kVec;
                 if (aligned && off + kVec <= count) {
                     u32x4 x = ldg<NT>((const u32x4*)(g + off));
@@ -408,7 +411,7 @@ __global__ __launch_bounds__(kNormBlock) void sumsq_partials_kernel(
             }
         } else {
             const float* g = (const float*)r.g;
-            for (int64_t done = 0; done < count; done += kGroup) {
+            for (int64_t done = 0; done < count; done += kNormGroup) {
                 const int64_t off = done + (int64_t)tid * kVec;
                 if (aligned && off + kVec <= count) {
                     f32x4 x0 = ldg<NT>((const f32x4*)(g + off)), x1 = ldg<NT>((const f32x4*)(g + off) + 1);
@@ -449,13 +452,13 @@ __global__ __launch_bounds__(kFinalBlock) void sumsq_final_kernel(
     const int tid = threadIdx.x;
     double a = 0.0;
     int64_t i = tid;
-    // eight independent loads in flight, added in index order: the same sum as one at a time
-    for (; i + 7 * (int64_t)kFinalBlock < n_partials; i += 8 * (int64_t)kFinalBlock) {
-        double x[8];
+    // sixteen independent loads in flight, added in index order: the same sum as one at a time
+    for (; i + 15 * (int64_t)kFinalBlock < n_partials; i += 16 * (int64_t)kFinalBlock) {
+        double x[16];
 #pragma unroll
-        for (int k = 0; k < 8; k++) x[k] = partials[i + k * (int64_t)kFinalBlock];
+        for (int k = 0; k < 16; k++) x[k] = partials[i + k * (int64_t)kFinalBlock];
 #pragma unroll
-        for (int k = 0; k < 8; k++) a += x[k];
+        for (int k = 0; k < 16; k++) a += x[k];
     }
     for (; i < n_partials; i += kFinalBlock) a += partials[i];
     acc[tid] = a;
@@ -476,7 +479,7 @@ __global__ __launch_bounds__(kFinalBlock) void sumsq_final_kernel(
 }
 
 // In-place scale of the gradients (trainer.h:136-145).  Exactly 1.0f: nothing is touched.
-__global__ __launch_bounds__(kNormBlock) void scale_grads_kernel(
+__global__ __launch_bounds__(kScaleBlock) void scale_grads_kernel(
     const ChunkRec* __restrict__ recs, int64_t n_chunks, const NormResult* __restrict__ norm)
 {
     const float scale = norm->scale;
@@ -873,7 +876,7 @@ int rlx_plan_norm_read(rlx_plan* p, float* norm, float* scale, double* sum_sq, v
 int rlx_plan_scale_grads(rlx_plan* p, void* stream) {
     if (!plan_ok(p)) return RLX_ERR_INVALID_ARG;
     int64_t g = p->n_chunks < kMaxNormGrid ? p->n_chunks : kMaxNormGrid;
-    scale_grads_kernel<<<dim3((unsigned)g), dim3(kNormBlock), 0, (hipStream_t)stream>>>(p->d_recs, p->n_chunks,
+    scale_grads_kernel<<<dim3((unsigned)g), dim3(kScaleBlock), 0, (hipStream_t)stream>>>(p->d_recs, p->n_chunks,
                                                                                       p->d_norm);
     RLX_HIP(hipGetLastError());
     return RLX_OK;
