@@ -11,11 +11,11 @@
 // Update kernel: a chunk is cut into tiles of 256 elements and every tile is one small
 // workgroup (128 lanes, two elements per lane: one 32-bit access per FP16 stream and one
 // 64-bit access per FP32 stream, each instruction contiguous across the wavefront, all
-// marked non-temporal, the stores also system-scope).  On MI355X this shape measured ~6.7 TB/s on the seven streams of
-// the update against ~5.3 TB/s for 128-bit accesses with several KB per workgroup: what
-// matters for a mixed read/write stream is that the set of addresses in flight stays a
-// narrow window, which many tiny workgroups dispatched in order give and fat workgroups or
-// grid-stride loops do not.  Consecutive workgroups go round-robin to the 8 XCDs; an optional
+// marked non-temporal, the stores also system-scope).  On MI355X this shape measured
+// ~6.8 TB/s on the seven streams of the update against ~5.3 TB/s for 128-bit accesses with
+// several KB per workgroup: what matters for a mixed read/write stream is that the set of
+// addresses in flight stays a narrow window, which many tiny workgroups dispatched in order
+// give and fat workgroups or grid-stride loops do not.  Consecutive workgroups go round-robin to the 8 XCDs; an optional
 // swizzle (K > 1) hands each XCD K neighbouring tiles, which did not pay in measurements.
 //
 // Norm kernel: one workgroup of 512 lanes per chunk with 128-bit reads; one FP64 partial
