@@ -141,3 +141,79 @@ def test_steps_reduce_a_loss(L, host, torch_gpu):
     losses.append(loss_and_grads())
     assert all(b < a for a, b in zip(losses, losses[1:])), losses
     assert opt.get_step() == 5
+
+
+def test_plans_can_be_created_and_destroyed_many_times(L, host, B, torch_gpu):
+    """A plan owns device tables, a workspace and pinned memory: 300 create / use / destroy rounds leave the
+    device's free memory where it was."""
+    torch = torch_gpu
+    specs = L.qwen3_tensor_list(MINI)
+    st = host.ParamStore(specs)
+    st.fill("g", 1, 0.0, 1e-3)
+    descs = st.descs()
+    torch.cuda.synchronize()
+    p = B.Plan(descs, 2048)
+    p.grad_norm(1.0)
+    first = p.norm_read()
+    p.destroy()
+    free0, _ = torch.cuda.mem_get_info()
+    for _ in range(300):
+        p = B.Plan(descs, 2048)
+        p.grad_norm(1.0)
+        assert p.norm_read() == first
+        p.destroy()
+    free1, _ = torch.cuda.mem_get_info()
+    assert abs(free0 - free1) < 8 * 2 ** 20
+    p.destroy()                                   # a second destroy of the wrapper is harmless
+
+
+def test_two_host_threads_with_their_own_plans_and_streams(O, L, host, B, torch_gpu):
+    """Two host threads step two optimizers on two streams at the same time; each result equals the
+    oracle's.  (One plan is not shared between threads: that is documented as unsupported.)"""
+    import threading
+    import numpy as np
+    from util import bits
+    torch = torch_gpu
+    specs = [L.TensorSpec("w", 300_000, L.DTYPE_F16, 0, 0), L.TensorSpec("n", 999, L.DTYPE_F32, L.NO_DECAY, 0)]
+    stores, opts, streams = [], [], [torch.cuda.Stream(), torch.cuda.Stream()]
+    for k in range(2):
+        s = host.ParamStore(specs)
+        s.fill("p", 1 + k, 0.0, 0.02)
+        s.fill("g", 3 + k, 0.0, 5e-3)
+        stores.append(s)
+        opts.append(host.AdamWOptimizer(s, lr=1e-3 * (k + 1)))
+    torch.cuda.synchronize()
+    before = [[(bits(s.param(i)), bits(s.grad(i))) for i in range(2)] for s in stores]
+    norms, errors = [None, None], []
+
+    def work(k):
+        try:
+            with torch.cuda.stream(streams[k]):
+                for _ in range(20):
+                    norms[k] = host.training_step(opts[k], 0.5, fused_clip=True)
+                streams[k].synchronize()
+        except Exception as exc:      # pragma: no cover
+            errors.append(exc)
+
+    threads = [threading.Thread(target=work, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    assert not errors, errors
+    for k in range(2):
+        hs = [dict(p=before[k][i][0], g=before[k][i][1], m=np.zeros(specs[i].n, np.float32),
+                   v=np.zeros(specs[i].n, np.float32)) for i in range(2)]
+        ssq, _ = O.sumsq_mirror([h["g"] for h in hs], opts[k].plan.chunk_elems)
+        scale, norm = O.clip_scale(np.float32(ssq), 0.5)
+        assert norms[k] == norm
+        for step in range(1, 21):
+            bc1, bc2 = host.bias_correction(0.9, step), host.bias_correction(0.999, step)
+            O.adamw_fp16(None, hs[0]["p"], hs[0]["g"], hs[0]["m"], hs[0]["v"], 1e-3 * (k + 1), 0.9, 0.999, 1e-8, 0.01,
+                         bc1, bc2, clip_scale=scale)
+            O.adamw_fp32(hs[1]["p"], hs[1]["g"], hs[1]["m"], hs[1]["v"], 1e-3 * (k + 1), 0.9, 0.999, 1e-8, 0.0,
+                         bc1, bc2, clip_scale=scale)
+        for i in range(2):
+            assert np.array_equal(bits(stores[k].param(i)), hs[i]["p"])
+            assert np.array_equal(bits(stores[k].state(i, "v")), hs[i]["v"])
