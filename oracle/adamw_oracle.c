@@ -296,19 +296,21 @@ float orc_clip_grad_norm(uint16_t* half_pool, int64_t n16, float* float_pool, in
 /* ------------------------------------------------------------------ */
 /* Mirror of the device reduction order (no counterpart in the         */
 /* reference).  A chunk is `chunk` consecutive elements of one tensor; */
-/* lane t of 512 owns the 8-element groups t, t+512, ... of the chunk  */
-/* and adds x*x into one FP32 accumulator in element order; the 64     */
-/* lanes of a wave combine by xor-butterfly (32,16,8,4,2,1); the eight */
-/* wave sums are added in FP64 in wave order.                          */
+/* with L = min(512, chunk/8) lanes, lane t owns the 8-element groups  */
+/* t, t+L, ... of the chunk and adds x*x into one FP32 accumulator in  */
+/* element order; the 64 lanes of a wave combine by xor-butterfly      */
+/* (32,16,8,4,2,1); the L/64 wave sums are added in FP64 in wave order.*/
 /* ------------------------------------------------------------------ */
 
 static double mirror_chunk(const void* g, int is_f32, int64_t count, int chunk)
 {
     float lane[512];
     int groups = chunk / 8;
-    for (int t = 0; t < 512; t++) {
+    int lanes = groups < 512 ? groups : 512;
+    if (lanes < 64) lanes = 64;
+    for (int t = 0; t < lanes; t++) {
         float acc = 0.0f;
-        for (int grp = t; grp < groups; grp += 512) {
+        for (int grp = t; grp < groups; grp += lanes) {
             for (int e = 0; e < 8; e++) {
                 int64_t i = (int64_t)grp * 8 + e;
                 if (i < count) {
@@ -320,7 +322,7 @@ static double mirror_chunk(const void* g, int is_f32, int64_t count, int chunk)
         lane[t] = acc;
     }
     double total = 0.0;
-    for (int w = 0; w < 8; w++) {
+    for (int w = 0; w < lanes / 64; w++) {
         float* l = lane + 64 * w;
         for (int mask = 32; mask >= 1; mask >>= 1) {
             float nxt[64];

@@ -39,10 +39,10 @@
 namespace {
 
 constexpr int kVec = 8;                       // elements per lane per group in the norm and scale passes
-constexpr int kNormBlock = 512;               // lanes per workgroup of the norm pass (8 wavefronts)
-constexpr int kNormGroup = kNormBlock * kVec; // 4096
+constexpr int kNormBlock = 512;               // most lanes per workgroup of the norm pass (8 wavefronts)
 constexpr int kScaleBlock = 256;              // lanes per workgroup of the scale pass
-constexpr int64_t kMinChunk = 2048;
+constexpr int64_t kMinChunk = 512;             // the largest tile of any update variant
+constexpr int64_t kSmallChunk = 2048;
 constexpr int64_t kBigChunk = 8192;
 constexpr int kFinalBlock = 1024;
 
@@ -349,18 +349,20 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
 
 // ---------------------------------------------------------------------------------------
 // Norm pass 1: one workgroup per chunk, one FP64 partial per chunk in the chunk's own slot.
-// Order inside a chunk (restated on the CPU by the test oracle): lane t of 512 adds x*x of its
-// 8-element groups t, t+512, ... element by element into one FP32 accumulator; the 64
-// lanes of a wavefront combine by xor butterfly with masks 32,16,8,4,2,1; the eight
+// BLOCK = min(512, chunk_elems / 8) lanes, so that small chunks do not launch idle wavefronts.
+// Order inside a chunk (restated on the CPU by the test oracle): lane t of BLOCK adds x*x of its
+// 8-element groups t, t+BLOCK, ... element by element into one FP32 accumulator; the 64
+// lanes of a wavefront combine by xor butterfly with masks 32,16,8,4,2,1; the BLOCK/64
 // wavefront sums go through LDS and are added in FP64 in wavefront order.  (512 lanes with
 // two 128-bit reads each measured 7.3 TB/s as a stand-alone stream, 256 lanes with four 6.95.)
 // ---------------------------------------------------------------------------------------
 
-template <bool NT>
-__global__ __launch_bounds__(kNormBlock) void sumsq_partials_kernel(
+template <bool NT, int BLOCK>
+__global__ __launch_bounds__(BLOCK) void sumsq_partials_kernel(
     const ChunkRec* __restrict__ recs, int64_t n_chunks, double* __restrict__ partials)
 {
-    __shared__ float wave_sum[kNormBlock / 64];
+    constexpr int kNormGroup = BLOCK * kVec;
+    __shared__ float wave_sum[BLOCK / 64];
     const int tid = threadIdx.x;
 
     for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
@@ -379,7 +381,7 @@ __global__ __launch_bounds__(kNormBlock) void sumsq_partials_kernel(
                     u32x4 x[2];
 #pragma unroll
                     for (int j = 0; j < 2; j++)
-                        x[j] = ldg<NT>((const u32x4*)(g + done + (int64_t)(j * kNormBlock + tid) * kVec));
+                        x[j] = ldg<NT>((const u32x4*)(g + done + (int64_t)(j * BLOCK + tid) * kVec));
 #pragma unroll
                     for (int j = 0; j < 2; j++) {
 #pragma unroll
@@ -434,7 +436,7 @@ __global__ __launch_bounds__(kNormBlock) void sumsq_partials_kernel(
         if (tid == 0) {
             double total = 0.0;
 #pragma unroll
-            for (int w = 0; w < kNormBlock / 64; w++) total += (double)wave_sum[w];
+            for (int w = 0; w < BLOCK / 64; w++) total += (double)wave_sum[w];
             partials[c] = total;
         }
         __syncthreads();
@@ -728,7 +730,8 @@ inline bool plan_ok(const rlx_plan* p) { return p && p->magic == kPlanMagic; }
 template <int BLOCK>
 void launch_scale_groups(const rlx_plan* p, hipStream_t s) {
     constexpr int TILE = BLOCK * kVec;
-    const int tpc_log2 = p->chunk_log2 - __builtin_ctz(TILE);
+    // chunks smaller than one group: one workgroup per chunk, the lanes beyond its end drop out
+    const int tpc_log2 = p->chunk_log2 > __builtin_ctz(TILE) ? p->chunk_log2 - __builtin_ctz(TILE) : 0;
     const int64_t n_tiles = p->n_chunks << tpc_log2;
     for (int64_t first = 0; first < n_tiles; first += kMaxTilesPerLaunch) {
         const int64_t here = n_tiles - first < kMaxTilesPerLaunch ? n_tiles - first : kMaxTilesPerLaunch;
@@ -795,7 +798,10 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
     }
     // Default: big chunks for big tensors; for a list of many small tensors a smaller chunk
     // wastes fewer workgroups on the empty part of each tensor's last chunk.
-    if (chunk_elems == 0) chunk_elems = n_elems / count >= 4 * kBigChunk ? kBigChunk : kMinChunk;
+    if (chunk_elems == 0) {
+        const int64_t mean = n_elems / count;
+        chunk_elems = mean >= 4 * kBigChunk ? kBigChunk : mean >= 4 * kSmallChunk ? kSmallChunk : kMinChunk;
+    }
     if (chunk_elems < kMinChunk || chunk_elems > (1 << 24) || (chunk_elems & (chunk_elems - 1)) != 0)
         return RLX_ERR_INVALID_ARG;
     int64_t n_chunks = 0;
@@ -864,11 +870,20 @@ int rlx_plan_grad_norm(rlx_plan* p, float max_norm, void* stream) {
     int64_t g = g_tuning.norm_grid > 0 ? g_tuning.norm_grid : p->n_chunks;
     if (g > p->n_chunks) g = p->n_chunks;
     if (g > kMaxNormGrid) g = kMaxNormGrid;
-    const dim3 grid((unsigned)g), block(kNormBlock);
-    if (g_tuning.norm_nt)
-        sumsq_partials_kernel<true><<<grid, block, 0, s>>>(p->d_recs, p->n_chunks, p->d_partials);
-    else
-        sumsq_partials_kernel<false><<<grid, block, 0, s>>>(p->d_recs, p->n_chunks, p->d_partials);
+    const dim3 grid((unsigned)g);
+    const int64_t lanes = p->chunk_elems / kVec < kNormBlock ? p->chunk_elems / kVec : kNormBlock;
+#define RLX_NORM_LAUNCH(BLOCK)                                                                                   \
+    do {                                                                                                         \
+        if (g_tuning.norm_nt)                                                                                    \
+            sumsq_partials_kernel<true, BLOCK><<<grid, dim3(BLOCK), 0, s>>>(p->d_recs, p->n_chunks, p->d_partials);  \
+        else                                                                                                     \
+            sumsq_partials_kernel<false, BLOCK><<<grid, dim3(BLOCK), 0, s>>>(p->d_recs, p->n_chunks, p->d_partials); \
+    } while (0)
+    if (lanes >= 512) RLX_NORM_LAUNCH(512);
+    else if (lanes == 256) RLX_NORM_LAUNCH(256);
+    else if (lanes == 128) RLX_NORM_LAUNCH(128);
+    else RLX_NORM_LAUNCH(64);
+#undef RLX_NORM_LAUNCH
     RLX_HIP(hipGetLastError());
     sumsq_final_kernel<<<dim3(1), dim3(kFinalBlock), 0, s>>>(p->d_partials, p->n_chunks, max_norm, p->d_norm);
     RLX_HIP(hipGetLastError());

@@ -71,7 +71,7 @@ def test_plan_argument_checks(B):
     assert lib.rlx_plan_create(None, 1, 0, C.byref(h)) == B.ERR_INVALID_ARG
     assert lib.rlx_plan_create(arr, 0, 0, C.byref(h)) == B.ERR_INVALID_ARG
     assert lib.rlx_plan_create(arr, 1, 3000, C.byref(h)) == B.ERR_INVALID_ARG        # not a power of two
-    assert lib.rlx_plan_create(arr, 1, 1024, C.byref(h)) == B.ERR_INVALID_ARG        # below 2048
+    assert lib.rlx_plan_create(arr, 1, 256, C.byref(h)) == B.ERR_INVALID_ARG         # below 512
     for bad in (B.TensorDesc(0x1000, 0x2000, 0x3000, 0x4000, None, 0, B.DTYPE_F16, 0),       # n == 0
                 B.TensorDesc(0x1000, None, 0x3000, 0x4000, None, 8, B.DTYPE_F16, 0),          # no gradient
                 B.TensorDesc(None, 0x2000, 0x3000, 0x4000, None, 8, B.DTYPE_F16, 0),          # no parameter
@@ -137,8 +137,8 @@ def test_plan_create_without_a_device_reports_an_error(B):
     d = B.TensorDesc(0x10000, 0x20000, 0x30000, 0x40000, None, 5000, B.DTYPE_F16, 0)
     st = lib.rlx_plan_create((B.TensorDesc * 1)(d), 1, 0, C.byref(h))
     if st == B.OK:
-        assert lib.rlx_plan_num_chunks(h) == 3 and lib.rlx_plan_num_elements(h) == 5000
-        assert lib.rlx_plan_chunk_elems(h) == 2048
+        assert lib.rlx_plan_num_chunks(h) == 10 and lib.rlx_plan_num_elements(h) == 5000
+        assert lib.rlx_plan_chunk_elems(h) == 512
         assert lib.rlx_plan_destroy(h) == B.OK
     else:
         assert st in (B.ERR_HIP, B.ERR_NO_DEVICE) and h.value is None

@@ -205,7 +205,7 @@ def test_ragged_list_equals_flat_tensor(O, L, host, B, torch_gpu):
     flat_m = torch.zeros(total, dtype=torch.float32, device="cuda:0")
     flat_v = torch.zeros(total, dtype=torch.float32, device="cuda:0")
     opt = host.AdamWOptimizer(st, lr=1e-5)
-    assert opt.plan.chunk_elems == 2048                      # small-tensor lists get small chunks
+    assert opt.plan.chunk_elems == 512                       # small-tensor lists get small chunks
     opt.step()
     bc1, bc2 = host.bias_correction(0.9, 1), host.bias_correction(0.999, 1)
     assert B.adamw_fp16(None, flat_p.data_ptr(), flat_g.data_ptr(), flat_m.data_ptr(), flat_v.data_ptr(), total,
@@ -229,7 +229,7 @@ def test_every_tile_shape_and_chunk_size_gives_the_same_bits(L, host, B, torch_g
              L.TensorSpec("c", 131, L.DTYPE_F16, L.NO_DECAY, 0)]
     results = []
     try:
-        for variant, chunk in [(0, 8192), (1, 8192), (2, 2048), (3, 2048), (4, 4096), (5, 65536), (6, 8192),
+        for variant, chunk in [(0, 8192), (1, 8192), (2, 2048), (3, 512), (4, 512), (5, 65536), (6, 1024),
                                (7, 2048)]:
             B.set_tuning("update_variant", variant)
             st = host.ParamStore(specs)
@@ -468,7 +468,7 @@ def test_random_plans(O, L, host, B, torch_gpu, seed):
     torch = torch_gpu
     rng = np.random.default_rng(1000 + seed)
     count = int(rng.integers(1, 14))
-    chunk = int(rng.choice([2048, 4096, 8192, 32768]))
+    chunk = int(rng.choice([512, 1024, 2048, 4096, 8192, 32768]))
     fused = bool(rng.integers(0, 2))
     zero = bool(rng.integers(0, 2))
     max_norm = float(rng.choice([0.0, 0.05, 1e6]))
