@@ -26,7 +26,9 @@ typedef enum {
     RLX_ERR_BAD_HYPER = 3,        /* bias correction of 0, or a non-finite hyper-parameter */
     RLX_ERR_HIP = 4,              /* a HIP runtime call failed; see rlx_last_hip_error() */
     RLX_ERR_NO_DEVICE = 5,
-    RLX_ERR_TOO_LARGE = 6         /* more chunks than one plan can address */
+    RLX_ERR_TOO_LARGE = 6,        /* more chunks than one plan can address */
+    RLX_ERR_NO_MEMORY = 7,        /* host allocation failed */
+    RLX_ERR_WRONG_DEVICE = 8      /* the plan was made with another device current */
 } rlx_status;
 
 const char* rlx_status_string(int status);
@@ -104,8 +106,8 @@ typedef struct rlx_plan rlx_plan;
  * Builds the device-resident work table for `count` tensors (the role that
  * AdamWOptimizer::init's offset bookkeeping has, include/training/optimizer.h:188-243).
  * Tensors are cut into chunks of `chunk_elems` elements (0 = chosen from the mean tensor
- * size: 8192, 2048 or 512; otherwise a power of two >= 512); the table order is the order of `descs`, which also fixes the
- * order of the norm reduction.  The plan borrows every pointer in `descs` and owns only
+ * size: 8192, 2048 or 512; otherwise a power of two >= 512); the table order is the order of
+ * `descs`, which also fixes the order of the norm reduction.  The plan borrows every pointer in `descs` and owns only
  * its tables and the reduction workspace.  Allocates; call outside the step loop.
  */
 int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_elems, rlx_plan** out);
@@ -122,7 +124,9 @@ int64_t rlx_plan_chunk_elems(const rlx_plan* plan);
  * a fixed order, so that the result is the same bits on every run.  Writes
  * {sum_sq, norm = sqrtf((float)sum_sq), scale} to the plan's device result, where
  * scale = max_norm / (norm + 1e-6f) iff norm > max_norm, else 1.0f (a NaN norm gives
- * 1.0f, as the reference's comparison does).  No host synchronisation.
+ * 1.0f, as the reference's comparison does; max_norm = INFINITY measures without clipping).
+ * No host synchronisation.  The plan must be used with the device current that it was
+ * created on (RLX_ERR_WRONG_DEVICE otherwise; the same holds for every launch below).
  */
 int rlx_plan_grad_norm(rlx_plan* plan, float max_norm, void* stream);
 

@@ -10,7 +10,8 @@ import os
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "librlx_adamw.so")
 
-OK, ERR_INVALID_ARG, ERR_MISALIGNED, ERR_BAD_HYPER, ERR_HIP, ERR_NO_DEVICE, ERR_TOO_LARGE = range(7)
+(OK, ERR_INVALID_ARG, ERR_MISALIGNED, ERR_BAD_HYPER, ERR_HIP, ERR_NO_DEVICE, ERR_TOO_LARGE, ERR_NO_MEMORY,
+ ERR_WRONG_DEVICE) = range(9)
 DTYPE_F16, DTYPE_F32 = 0, 1
 TENSOR_NO_DECAY, TENSOR_GRAD_ONLY, TENSOR_FROZEN = 1, 2, 4
 CLIP_NONE, CLIP_FUSED, STEP_ZERO_GRADS = 0, 1, 2

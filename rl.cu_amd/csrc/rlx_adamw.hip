@@ -15,10 +15,11 @@
 // ~6.8 TB/s on the seven streams of the update against ~5.3 TB/s for 128-bit accesses with
 // several KB per workgroup: what matters for a mixed read/write stream is that the set of
 // addresses in flight stays a narrow window, which many tiny workgroups dispatched in order
-// give and fat workgroups or grid-stride loops do not.  Consecutive workgroups go round-robin to the 8 XCDs; an optional
-// swizzle (K > 1) hands each XCD K neighbouring tiles, which did not pay in measurements.
+// give and fat workgroups or grid-stride loops do not.  Consecutive workgroups go round-robin
+// to the 8 XCDs; an optional swizzle (K > 1) hands each XCD K neighbouring tiles, which did
+// not pay in measurements.
 //
-// Norm kernel: one workgroup of 512 lanes per chunk with 128-bit reads; one FP64 partial
+// Norm kernel: one workgroup of up to 512 lanes per chunk with 128-bit reads; one FP64 partial
 // per chunk in a fixed slot, then a single-workgroup pass in fixed order (no atomics).
 //
 // Arithmetic follows src/kernels/adamw.cu:25-39 of the reference operation by operation
@@ -513,7 +514,15 @@ __global__ __launch_bounds__(BLOCK) void scale_group_kernel(
         }
     } else {
         float* g = (float*)r.g;
-        for (int64_t i = off; i < off + kVec && i < count; i++) g[i] = g[i] * scale;
+        if (aligned && off + kVec <= count) {
+            f32x4 x0 = ldg<true>((const f32x4*)(g + off)), x1 = ldg<true>((const f32x4*)(g + off) + 1);
+#pragma unroll
+            for (int k = 0; k < 4; k++) { x0[k] = x0[k] * scale; x1[k] = x1[k] * scale; }
+            st_stream<1>((f32x4*)(g + off), x0);
+            st_stream<1>((f32x4*)(g + off) + 1, x1);
+        } else {
+            for (int64_t i = off; i < off + kVec && i < count; i++) g[i] = g[i] * scale;
+        }
     }
 }
 
@@ -652,8 +661,6 @@ ChunkRec make_rec(const rlx_tensor_desc& d, int64_t start, int64_t count) {
     return r;
 }
 
-struct UpdateVariant { int tile; };
-
 template <int E, int BLOCK, int K, bool SINGLE, int SP>
 void launch_variant(const ChunkRec* recs, const ChunkRec& single, int64_t single_n, int64_t n_elems_or_tiles,
                     int chunk_log2, const Hyper& h, const rlx_step_params* dev_params, const NormResult* norm,
@@ -727,6 +734,15 @@ namespace {
 constexpr uint32_t kPlanMagic = 0x524C5850u;   // "RLXP"
 inline bool plan_ok(const rlx_plan* p) { return p && p->magic == kPlanMagic; }
 
+// A plan's tables and every pointer in them belong to the device that was current when the plan
+// was made; launching it with another device current would hand that device foreign addresses.
+int plan_launchable(const rlx_plan* p) {
+    if (!plan_ok(p)) return RLX_ERR_INVALID_ARG;
+    int dev = -1;
+    RLX_HIP(hipGetDevice(&dev));
+    return dev == p->device ? RLX_OK : RLX_ERR_WRONG_DEVICE;
+}
+
 template <int BLOCK>
 void launch_scale_groups(const rlx_plan* p, hipStream_t s) {
     constexpr int TILE = BLOCK * kVec;
@@ -753,13 +769,15 @@ const char* rlx_status_string(int status) {
     case RLX_ERR_HIP: return "HIP runtime error";
     case RLX_ERR_NO_DEVICE: return "no HIP device";
     case RLX_ERR_TOO_LARGE: return "too many chunks for one plan";
+    case RLX_ERR_NO_MEMORY: return "out of host memory";
+    case RLX_ERR_WRONG_DEVICE: return "the plan belongs to another device than the current one";
     default: return "unknown status";
     }
 }
 
 const char* rlx_last_hip_error(void) { return g_hip_error; }
 
-int rlx_version(void) { return 101; }
+int rlx_version(void) { return 102; }
 
 int rlx_adamw_fp16(float* master_w, uint16_t* model_w, const uint16_t* grad, float* m, float* v, int64_t n,
                    float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -809,7 +827,11 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
     if (n_chunks > INT32_MAX) return RLX_ERR_TOO_LARGE;
 
     std::vector<ChunkRec> recs;
-    recs.reserve((size_t)n_chunks);
+    try {
+        recs.reserve((size_t)n_chunks);
+    } catch (const std::bad_alloc&) {
+        return RLX_ERR_NO_MEMORY;
+    }
     for (int64_t i = 0; i < count; i++) {
         for (int64_t start = 0; start < descs[i].n; start += chunk_elems) {
             const int64_t left = descs[i].n - start;
@@ -818,7 +840,7 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
     }
 
     rlx_plan* p = new (std::nothrow) rlx_plan();
-    if (!p) return RLX_ERR_INVALID_ARG;
+    if (!p) return RLX_ERR_NO_MEMORY;
     p->magic = kPlanMagic;
     p->chunk_log2 = __builtin_ctzll((unsigned long long)chunk_elems);
     p->n_tensors = count; p->n_chunks = n_chunks; p->n_elems = n_elems; p->chunk_elems = chunk_elems;
@@ -865,7 +887,8 @@ const void* rlx_plan_norm_device_ptr(const rlx_plan* p) { return plan_ok(p) ? p-
 const double* rlx_plan_partials_device_ptr(const rlx_plan* p) { return plan_ok(p) ? p->d_partials : nullptr; }
 
 int rlx_plan_grad_norm(rlx_plan* p, float max_norm, void* stream) {
-    if (!plan_ok(p)) return RLX_ERR_INVALID_ARG;
+    const int ready = plan_launchable(p);
+    if (ready != RLX_OK) return ready;
     hipStream_t s = (hipStream_t)stream;
     int64_t g = g_tuning.norm_grid > 0 ? g_tuning.norm_grid : p->n_chunks;
     if (g > p->n_chunks) g = p->n_chunks;
@@ -891,7 +914,8 @@ int rlx_plan_grad_norm(rlx_plan* p, float max_norm, void* stream) {
 }
 
 int rlx_plan_norm_read(rlx_plan* p, float* norm, float* scale, double* sum_sq, void* stream) {
-    if (!plan_ok(p)) return RLX_ERR_INVALID_ARG;
+    const int ready = plan_launchable(p);
+    if (ready != RLX_OK) return ready;
     hipStream_t s = (hipStream_t)stream;
     RLX_HIP(hipMemcpyAsync(p->h_norm, p->d_norm, sizeof(NormResult), hipMemcpyDeviceToHost, s));
     RLX_HIP(hipStreamSynchronize(s));
@@ -902,7 +926,8 @@ int rlx_plan_norm_read(rlx_plan* p, float* norm, float* scale, double* sum_sq, v
 }
 
 int rlx_plan_scale_grads(rlx_plan* p, void* stream) {
-    if (!plan_ok(p)) return RLX_ERR_INVALID_ARG;
+    const int ready = plan_launchable(p);
+    if (ready != RLX_OK) return ready;
     launch_scale_groups<kScaleBlock>(p, (hipStream_t)stream);
     RLX_HIP(hipGetLastError());
     return RLX_OK;
@@ -911,6 +936,8 @@ int rlx_plan_scale_grads(rlx_plan* p, void* stream) {
 int rlx_plan_adamw(rlx_plan* p, const rlx_step_params* sp, int step_flags, void* stream) {
     if (!plan_ok(p) || !sp) return RLX_ERR_INVALID_ARG;
     if (step_flags & ~(RLX_CLIP_FUSED | RLX_STEP_ZERO_GRADS)) return RLX_ERR_INVALID_ARG;
+    const int ready = plan_launchable(p);
+    if (ready != RLX_OK) return ready;
     int st = check_hyper(sp->lr, sp->beta1, sp->beta2, sp->eps, sp->weight_decay, sp->bias_correction1,
                          sp->bias_correction2);
     if (st != RLX_OK) return st;
@@ -927,6 +954,8 @@ int rlx_plan_adamw_dev(rlx_plan* p, const rlx_step_params* dev_params, int step_
     if (!plan_ok(p) || !dev_params) return RLX_ERR_INVALID_ARG;
     if (step_flags & ~(RLX_CLIP_FUSED | RLX_STEP_ZERO_GRADS)) return RLX_ERR_INVALID_ARG;
     if (!is_aligned(dev_params, 4)) return RLX_ERR_MISALIGNED;
+    const int ready = plan_launchable(p);
+    if (ready != RLX_OK) return ready;
     ChunkRec none;
     memset(&none, 0, sizeof(none));
     Hyper h;

@@ -41,7 +41,7 @@ def test_version_and_status_strings(B):
     lib = B.load()
     assert lib.rlx_version() >= 100
     assert lib.rlx_status_string(B.OK) == b"ok"
-    for st in range(1, 7):
+    for st in range(1, B.ERR_WRONG_DEVICE + 1):
         assert lib.rlx_status_string(st) not in (b"ok", b"unknown status")
     assert lib.rlx_status_string(99) == b"unknown status"
 
