@@ -9,6 +9,10 @@ timed too and reported under "clip_step".
 
 Prints ONE JSON line.  The CPU oracle is used here only as the checker of a sample and as the
 timed CPU baseline.
+
+--workload selects one of the other configurations instead (flat-1m, qwen3-0.6b-master, ragged,
+qwen3-8b): the same kind of line with fewer legs (update, norm, norm + fused-clip update; seeded
+state, no oracle replay: the GPU tests hold the parity of these configurations).
 """
 import argparse
 import importlib
@@ -63,11 +67,95 @@ def cpu_baseline(O, host, sample, hyper, step, seconds=8.0):
             "gbps": BYTES_UPDATE * p.size * reps / el / 1e9}
 
 
+def time_events(fn, warmup, steps):
+    """ms per call: `steps` calls back to back between two events on torch's current stream."""
+    import torch
+    for _ in range(warmup):
+        fn()
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(steps):
+        fn()
+    b.record()
+    torch.cuda.synchronize()
+    return a.elapsed_time(b) / steps
+
+
+def other_workload(args, pkg, host):
+    """Update, norm and norm + fused-clip update of one of the secondary configurations."""
+    import torch
+    B, L = pkg.binding, pkg.layout
+    name, master, extra = args.workload, False, {}
+    if name == "flat-1m":
+        specs = [L.TensorSpec("flat", 1 << 20, L.DTYPE_F16, 0, 0)]
+        p_std, g_std, what = 0.02, 1e-3, "one flat tensor of 1,048,576 FP16 parameters (22 MB: cache-resident)"
+    elif name == "qwen3-0.6b-master":
+        specs = L.qwen3_tensor_list(L.QWEN3_0_6B, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
+        master, p_std, g_std = True, 0.02, 5e-3
+        what = "Qwen3-0.6B in the reference's layout: FP32 norm weights, FP32 master copy, no decay on embedding and norms"
+    elif name == "ragged":
+        specs = L.ragged_tensor_list()
+        p_std, g_std, what = 0.01, 1e-3, "4,096 tensors of 128..65,536 elements in one launch (cache-resident)"
+    elif name == "qwen3-8b":
+        specs = L.qwen3_tensor_list(L.QWEN3_8B)
+        p_std, g_std, what = 0.02, 1e-4, "Qwen3-8B tensor list, untied lm_head, 98 GB resident, step 1000, clip active"
+    else:
+        raise SystemExit("unknown workload " + name)
+    N = L.total_elements(specs)
+    st = host.ParamStore(specs, "cuda:0", master=master)
+    st.fill("p", SEED_P, 1.0 if name == "ragged" else 0.0, p_std)
+    st.fill("g", SEED_G, 0.0, g_std)
+    st.fill("m", SEED_P + 1, 0.0, 1e-4)
+    st.fill("v", SEED_P + 2, 1e-8, 1e-8, flags=B.FILL_ABS)
+    if master:
+        st.init_master()
+    opt = host.AdamWOptimizer(st, lr=1e-5, chunk_elems=args.chunk)
+    opt.step_ = 999
+    stream = torch.cuda.current_stream().cuda_stream
+    bpp = 28 if master else BYTES_UPDATE
+    steps, warm = args.steps, args.warmup
+    upd = time_events(lambda: opt.step(), warm, steps)
+    nrm = time_events(lambda: opt.plan.grad_norm(1.0, stream), warm, steps)
+
+    def clip_step():
+        opt.plan.grad_norm(1.0, stream)
+        opt.step(fused_clip=True)
+
+    both = time_events(clip_step, warm, steps)
+    norm, scale, _ = opt.plan.norm_read(stream)
+    if name == "ragged":      # against one flat tensor of the same element count
+        flat = host.ParamStore([L.TensorSpec("flat", N, L.DTYPE_F16, 0, 0)], "cuda:0")
+        fopt = host.AdamWOptimizer(flat, lr=1e-5)
+        extra["flat_tensor_same_count_ms"] = time_events(lambda: fopt.step(), warm, steps)
+    gbps = bpp * N / (upd * 1e-3) / 1e9
+    out = {
+        "metric": "AdamW params/sec, %s step" % name, "value": N / (upd * 1e-3), "unit": "params/s",
+        "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": upd, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": what, "params": N, "tensors": len(specs), "bytes_per_param": bpp,
+                   "chunk_elems": opt.plan.chunk_elems, "chunks": opt.plan.num_chunks,
+                   "update_variant": B.get_tuning("update_variant")},
+        "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "kernel_ms": upd,
+                     "algorithmic_bytes_per_launch": bpp * N},
+        "cpu_baseline": None,
+        "norm_ms": nrm, "norm_gbps": BYTES_NORM * N / (nrm * 1e-3) / 1e9,
+        "clip_step": {"ms_per_step": both, "achieved_gbps": (bpp + BYTES_NORM) * N / (both * 1e-3) / 1e9,
+                      "grad_norm": norm, "clip_scale": scale},
+    }
+    out.update(extra)
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="qwen3-0.6b",
+                    help="qwen3-0.6b (default, the headline), flat-1m, qwen3-0.6b-master, ragged, qwen3-8b")
+    ap.add_argument("--chunk", type=int, default=0, help="chunk_elems of the plan (0 = automatic)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--variant", type=int, default=None, help="update kernel tile shape (tuning)")
     ap.add_argument("--quick-setup", action="store_true",
@@ -92,6 +180,9 @@ def main():
     O = entry.load_oracle()
     if args.variant is not None:
         B.set_tuning("update_variant", args.variant)
+    if args.workload != "qwen3-0.6b":
+        other_workload(args, pkg, host)
+        return
 
     hyper = dict(lr=1e-5, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01)
     specs = L.qwen3_tensor_list(L.QWEN3_0_6B)
@@ -99,7 +190,7 @@ def main():
     st = host.ParamStore(specs, "cuda:0")
     st.fill("p", SEED_P, 0.0, 0.02)
     opt = host.AdamWOptimizer(st, lr=hyper["lr"], beta1=hyper["beta1"], beta2=hyper["beta2"], eps=hyper["eps"],
-                              weight_decay=hyper["wd"])
+                              weight_decay=hyper["wd"], chunk_elems=args.chunk)
     emb = [i for i, s in enumerate(specs) if s.name == "embed_tokens"][0]
 
     # ---- parity of a sample while the state is built: 99 seeded steps, oracle replays a slice ----
