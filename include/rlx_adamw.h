@@ -111,6 +111,15 @@ typedef struct rlx_plan rlx_plan;
  * its tables and the reduction workspace.  Allocates; call outside the step loop.
  */
 int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_elems, rlx_plan** out);
+/*
+ * The chunking that rlx_plan_create would use for these arguments, computed on the host without
+ * touching a device: the chunk size (the chosen one if chunk_elems is 0), the number of chunks
+ * (= device records = FP64 partials of the norm) and the number of elements.  Any out pointer may
+ * be NULL.  Same argument checks and status codes as rlx_plan_create.  No counterpart in the
+ * reference, whose launches are sized from flat pool lengths (include/training/optimizer.h:124-146).
+ */
+int rlx_plan_layout(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_elems, int64_t* out_chunk_elems,
+                    int64_t* out_num_chunks, int64_t* out_num_elements);
 int rlx_plan_destroy(rlx_plan* plan);
 int64_t rlx_plan_num_chunks(const rlx_plan* plan);
 int64_t rlx_plan_num_elements(const rlx_plan* plan);

@@ -46,6 +46,7 @@ SIGNATURES = {
     "rlx_adamw_fp32": ([_VP, _VP, _VP, _VP, _I64] + _HYPER + [_VP], _INT),
     "rlx_fp16_to_fp32": ([_VP, _VP, _I64, _VP], _INT),
     "rlx_plan_create": ([C.POINTER(TensorDesc), _I64, _I64, C.POINTER(_VP)], _INT),
+    "rlx_plan_layout": ([C.POINTER(TensorDesc), _I64, _I64, C.POINTER(_I64), C.POINTER(_I64), C.POINTER(_I64)], _INT),
     "rlx_plan_destroy": ([_VP], _INT),
     "rlx_plan_num_chunks": ([_VP], _I64),
     "rlx_plan_num_elements": ([_VP], _I64),
@@ -140,6 +141,15 @@ def fill_f16(dst, n, seed, mean, std, first=0, flags=0, row_len=0, zero_rows_bel
 def fill_f32(dst, n, seed, mean, std, first=0, flags=0, row_len=0, zero_rows_below=0, stream=0):
     check(load().rlx_fill_f32(dst, n, seed, first, mean, std, flags, row_len, zero_rows_below, stream),
           "rlx_fill_f32")
+
+
+def plan_layout(descs, chunk_elems=0):
+    """(chunk_elems, num_chunks, num_elements) that a plan over `descs` would have; host only."""
+    arr = (TensorDesc * len(descs))(*descs)
+    ce, nc, ne = _I64(), _I64(), _I64()
+    check(load().rlx_plan_layout(arr, len(descs), chunk_elems, C.byref(ce), C.byref(nc), C.byref(ne)),
+          "rlx_plan_layout")
+    return ce.value, nc.value, ne.value
 
 
 class Plan:

@@ -777,7 +777,7 @@ const char* rlx_status_string(int status) {
 
 const char* rlx_last_hip_error(void) { return g_hip_error; }
 
-int rlx_version(void) { return 102; }
+int rlx_version(void) { return 103; }
 
 int rlx_adamw_fp16(float* master_w, uint16_t* model_w, const uint16_t* grad, float* m, float* v, int64_t n,
                    float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -804,9 +804,8 @@ int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream) {
     return RLX_OK;
 }
 
-int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_elems, rlx_plan** out) {
-    if (!out) return RLX_ERR_INVALID_ARG;
-    *out = nullptr;
+int rlx_plan_layout(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_elems, int64_t* out_chunk_elems,
+                    int64_t* out_num_chunks, int64_t* out_num_elements) {
     if (!descs || count <= 0 || count > INT32_MAX) return RLX_ERR_INVALID_ARG;
     int64_t n_elems = 0;
     for (int64_t i = 0; i < count; i++) {
@@ -825,6 +824,18 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
     int64_t n_chunks = 0;
     for (int64_t i = 0; i < count; i++) n_chunks += (descs[i].n + chunk_elems - 1) / chunk_elems;
     if (n_chunks > INT32_MAX) return RLX_ERR_TOO_LARGE;
+    if (out_chunk_elems) *out_chunk_elems = chunk_elems;
+    if (out_num_chunks) *out_num_chunks = n_chunks;
+    if (out_num_elements) *out_num_elements = n_elems;
+    return RLX_OK;
+}
+
+int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_elems, rlx_plan** out) {
+    if (!out) return RLX_ERR_INVALID_ARG;
+    *out = nullptr;
+    int64_t n_elems = 0, n_chunks = 0;
+    const int layout = rlx_plan_layout(descs, count, chunk_elems, &chunk_elems, &n_chunks, &n_elems);
+    if (layout != RLX_OK) return layout;
 
     std::vector<ChunkRec> recs;
     try {

@@ -143,3 +143,44 @@ def test_plan_create_without_a_device_reports_an_error(B):
     else:
         assert st in (B.ERR_HIP, B.ERR_NO_DEVICE) and h.value is None
         assert lib.rlx_last_hip_error() != b""
+
+
+def test_plan_layout_on_the_host(B, L):
+    """Chunk size rule and chunk counts, computed without a device (include/rlx_adamw.h: rlx_plan_layout)."""
+    def descs(sizes, dtype=None):
+        out, at = [], 0x100000
+        for n in sizes:
+            out.append(B.TensorDesc(at, at + (1 << 40), at + (2 << 40), at + (3 << 40), None, n,
+                                    B.DTYPE_F16 if dtype is None else dtype, 0))
+            at += (n * 4 + 255) // 256 * 256
+        return out
+    # the automatic chunk follows the mean tensor size: 8192 from 32 Ki elements, 2048 from 8 Ki, else 512
+    assert B.plan_layout(descs([32768]))[0] == 8192
+    assert B.plan_layout(descs([32767]))[0] == 2048
+    assert B.plan_layout(descs([8192]))[0] == 2048
+    assert B.plan_layout(descs([8191]))[0] == 512
+    assert B.plan_layout(descs([1]))[:2] == (512, 1)
+    assert B.plan_layout(descs([100000, 128]))[0] == 8192          # mean 50,064
+    # chunk count = sum of per-tensor ceilings; a tensor never shares a chunk with its neighbour
+    sizes = [1, 511, 512, 513, 70000]
+    for chunk in (512, 1024, 8192, 1 << 24):
+        ce, nc, ne = B.plan_layout(descs(sizes), chunk)
+        assert ce == chunk and ne == sum(sizes) and nc == sum(-(-n // chunk) for n in sizes)
+    # the workloads of the benchmark
+    q = L.qwen3_tensor_list(L.QWEN3_0_6B)
+    assert B.plan_layout(descs([t.n for t in q])) == (8192, 72865, 596_049_920)
+    r = L.ragged_tensor_list()
+    ce, nc, ne = B.plan_layout(descs([t.n for t in r]))
+    assert ce == 512 and ne == L.total_elements(r) and nc == sum(-(-t.n // 512) for t in r)
+    big = L.qwen3_tensor_list(L.QWEN3_8B)
+    assert B.plan_layout(descs([t.n for t in big]))[:2] == (8192, 999_953)
+    # same argument checks as rlx_plan_create
+    lib = B.load()
+    arr = (B.TensorDesc * 1)(*descs([5000]))
+    assert lib.rlx_plan_layout(arr, 1, 3000, None, None, None) == B.ERR_INVALID_ARG
+    assert lib.rlx_plan_layout(arr, 1, 256, None, None, None) == B.ERR_INVALID_ARG
+    assert lib.rlx_plan_layout(arr, 1, 1 << 25, None, None, None) == B.ERR_INVALID_ARG
+    assert lib.rlx_plan_layout(None, 1, 0, None, None, None) == B.ERR_INVALID_ARG
+    assert lib.rlx_plan_layout(arr, 1, 0, None, None, None) == B.OK
+    huge = (B.TensorDesc * 1)(B.TensorDesc(0x1000, 0x2000, 0x3000, 0x4000, None, 1 << 41, B.DTYPE_F16, 0))
+    assert lib.rlx_plan_layout(huge, 1, 512, None, None, None) == B.ERR_TOO_LARGE
