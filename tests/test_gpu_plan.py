@@ -551,3 +551,25 @@ def test_random_plans(O, L, host, B, torch_gpu, seed):
         for d, h in zip(tensors, host_side):
             h["g"] = bits(d["g"])
     plan.destroy()
+
+
+@pytest.mark.gpu
+def test_plan_refuses_to_launch_on_another_device(B):
+    """A plan's tables belong to the device that was current when it was made."""
+    import torch
+    if torch.cuda.device_count() < 2:
+        pytest.skip("needs two devices")
+    n = 4096
+    with torch.cuda.device(0):
+        p = torch.zeros(n, dtype=torch.float16, device="cuda:0"); g = torch.zeros_like(p)
+        m = torch.zeros(n, dtype=torch.float32, device="cuda:0"); v = torch.zeros_like(m)
+        plan = B.Plan([B.TensorDesc(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), None, n, B.DTYPE_F16, 0)])
+    lib = B.load()
+    sp = B.StepParams(1e-3, 0.9, 0.999, 1e-8, 0.0, 0.1, 0.001)
+    with torch.cuda.device(1):
+        assert lib.rlx_plan_adamw(plan._h, sp, 0, None) == B.ERR_WRONG_DEVICE
+        assert lib.rlx_plan_grad_norm(plan._h, 1.0, None) == B.ERR_WRONG_DEVICE
+        assert lib.rlx_plan_scale_grads(plan._h, None) == B.ERR_WRONG_DEVICE
+    with torch.cuda.device(0):
+        assert lib.rlx_plan_adamw(plan._h, sp, 0, None) == B.OK
+        torch.cuda.synchronize()
