@@ -184,3 +184,79 @@ def test_against_frozen_vectors(B, host, torch_gpu):
         torch.cuda.synchronize()
         assert bits(w).view(np.uint32).tolist() == s["w"] and bits(m32).view(np.uint32).tolist() == s["m"]
         assert bits(v32).view(np.uint32).tolist() == s["v"]
+
+
+@pytest.mark.parametrize("eps,wd", [(1e-8, 0.01), (0.0, 0.0)])
+@pytest.mark.parametrize("with_master", [False, True])
+def test_every_half_gradient_against_special_moments(O, B, host, torch_gpu, eps, wd, with_master):
+    """Every FP16 bit pattern as the gradient (zeros, subnormals, infinities, NaNs) crossed with FP32 moments
+    and weights at the edges of the format: zero, negative zero, subnormal, the smallest and largest normal
+    numbers, infinity, NaN, and a negative second moment.  IEEE division and square root, kept denormals and
+    the final rounding to FP16 must give the oracle's bits; a NaN must meet a NaN (payloads are not compared)."""
+    torch = torch_gpu
+    f32 = np.float32
+    m_set = np.array([0.0, -0.0, 1e-45, -3e-39, 1.17549435e-38, 1e-3, -7.5, 3.4e38, np.inf, -np.inf, np.nan], f32)
+    v_set = np.array([0.0, 1e-45, 2e-39, 1.17549435e-38, 1e-20, 1e-6, 4.0, 3.4e38, np.inf, np.nan, -1e-6], f32)
+    p_set = np.array([0x0000, 0x8000, 0x0001, 0x03FF, 0x0400, 0x2E66, 0xBC00, 0x7BFF, 0x7C00, 0x7E00], np.uint16)
+    g_all = np.arange(65536, dtype=np.uint16)
+    reps = len(m_set) * len(v_set)
+    g_h = np.tile(g_all, reps)
+    m_h = np.repeat(np.tile(m_set, len(v_set)), 65536).astype(f32)
+    v_h = np.repeat(np.repeat(v_set, len(m_set)), 65536).astype(f32)
+    n = g_h.size
+    p_h = p_set[(np.arange(n) // 7) % len(p_set)].copy()
+    w_h = O.h2f(p_h) if with_master else None
+
+    def dev(a):
+        t = torch.from_numpy(a.view(np.int16) if a.dtype == np.uint16 else a).to("cuda:0")
+        return t.view(torch.float16) if a.dtype == np.uint16 else t
+
+    g_d, m_d, v_d, p_d = dev(g_h), dev(m_h), dev(v_h), dev(p_h)
+    w_d = dev(w_h) if with_master else None
+    bc1, bc2 = host.bias_correction(0.9, 3), host.bias_correction(0.999, 3)
+    args = (1e-3, 0.9, 0.999, eps, wd, bc1, bc2)
+    assert B.adamw_fp16(w_d.data_ptr() if with_master else None, p_d.data_ptr(), g_d.data_ptr(), m_d.data_ptr(),
+                        v_d.data_ptr(), n, *args) == B.OK
+    O.adamw_fp16(w_h, p_h, g_h, m_h, v_h, *args)
+    torch.cuda.synchronize()
+
+    def same(got, exp, what):
+        if got.dtype == np.uint16:
+            nan_g, nan_e = (got & 0x7FFF) > 0x7C00, (exp & 0x7FFF) > 0x7C00
+            eq = got == exp
+        else:
+            nan_g, nan_e = np.isnan(got), np.isnan(exp)
+            eq = got.view(np.uint32) == exp.view(np.uint32)
+        bad = ~(eq | (nan_g & nan_e))
+        assert not bad.any(), "%s: %d differ, first at %d: got %r expected %r" % (
+            what, int(bad.sum()), int(np.argmax(bad)), got[np.argmax(bad)], exp[np.argmax(bad)])
+        return int(nan_e.sum())
+
+    nans = same(bits(p_d), p_h, "p") + same(bits(m_d), m_h, "m") + same(bits(v_d), v_h, "v")
+    if with_master:
+        same(bits(w_d), w_h, "master")
+    assert nans > 0          # the grid does reach the non-finite cases
+
+
+def test_fp32_update_on_random_bit_patterns(O, B, host, torch_gpu):
+    """Four million elements whose weight, gradient and moments are uniformly random 32-bit patterns (every
+    exponent, subnormals, infinities, NaNs, negative second moments): the FP32 update gives the oracle's bits
+    wherever the oracle's result is a number, and a NaN wherever it is a NaN."""
+    torch = torch_gpu
+    n = 1 << 22
+    rng = np.random.default_rng(20240607)
+    host_arrays = [rng.integers(0, 1 << 32, n, dtype=np.uint64).astype(np.uint32).view(np.float32) for _ in range(4)]
+    w_h, g_h, m_h, v_h = host_arrays
+    w_d, g_d, m_d, v_d = [torch.from_numpy(a.copy()).to("cuda:0") for a in host_arrays]
+    bc1, bc2 = host.bias_correction(0.9, 7), host.bias_correction(0.999, 7)
+    args = (1e-3, 0.9, 0.999, 1e-8, 0.01, bc1, bc2)
+    assert B.adamw_fp32(w_d.data_ptr(), g_d.data_ptr(), m_d.data_ptr(), v_d.data_ptr(), n, *args) == B.OK
+    O.adamw_fp32(w_h, g_h, m_h, v_h, *args)
+    torch.cuda.synchronize()
+    finite = 0
+    for got, exp, what in ((bits(w_d), w_h, "w"), (bits(m_d), m_h, "m"), (bits(v_d), v_h, "v")):
+        nan_g, nan_e = np.isnan(got), np.isnan(exp)
+        bad = ~((got.view(np.uint32) == exp.view(np.uint32)) | (nan_g & nan_e))
+        assert not bad.any(), "%s: %d differ, first at %d" % (what, int(bad.sum()), int(np.argmax(bad)))
+        finite += int(np.isfinite(exp).sum())
+    assert finite > n        # most results are numbers, not NaN

@@ -189,6 +189,42 @@ def test_non_finite_gradient(O, L, host, torch_gpu):
     assert np.isnan(p[1234]) and np.isfinite(np.delete(p, 1234)).all()
 
 
+@pytest.mark.parametrize("fused", [False, True])
+def test_infinite_gradient(O, L, host, torch_gpu, fused):
+    """An infinite gradient gives an infinite norm and the scale max/(inf + 1e-6f) = 0
+    (include/training/trainer.h:343-344): every finite gradient becomes a (signed) zero, the infinite one
+    0 * inf = NaN, with the scale pass and fused alike; the oracle's two-step restatement agrees bit for bit
+    on every finite result."""
+    torch = torch_gpu
+    n = 5000
+    specs = [L.TensorSpec("a", n, L.DTYPE_F16, 0, 0)]
+    st = host.ParamStore(specs)
+    st.fill("p", 1, 0.0, 0.02)
+    st.fill("g", 2, 0.0, 1e-2)
+    st.grad(0)[777] = float("inf")
+    torch.cuda.synchronize()
+    p_h, g_h = bits(st.param(0)), bits(st.grad(0))
+    m_h, v_h = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    opt = host.AdamWOptimizer(st, lr=1e-3)
+    norm = host.training_step(opt, 1.0, fused_clip=fused)
+    torch.cuda.synchronize()
+    _, scale, _ = opt.plan.norm_read()
+    assert np.isinf(norm) and scale == 0.0
+    assert O.clip_scale(float("inf"), 1.0) == (0.0, float("inf"))
+    O.scale_half(g_h, 0.0)
+    O.adamw_fp16(None, p_h, g_h, m_h, v_h, 1e-3, 0.9, 0.999, 1e-8, 0.01, host.bias_correction(0.9, 1),
+                 host.bias_correction(0.999, 1))
+    got_p, got_m, got_v = bits(st.param(0)), bits(st.state(0, "m")), bits(st.state(0, "v"))
+    keep = np.arange(n) != 777
+    assert np.array_equal(got_p[keep], p_h[keep])
+    assert np.array_equal(got_m[keep].view(np.uint32), m_h[keep].view(np.uint32))
+    assert np.array_equal(got_v[keep].view(np.uint32), v_h[keep].view(np.uint32))
+    assert np.isnan(got_m[777]) and np.isnan(m_h[777]) and (got_p[777] & 0x7FFF) > 0x7C00
+    if not fused:
+        g_after = bits(st.grad(0))
+        assert np.array_equal(g_after[keep], g_h[keep]) and (g_after[777] & 0x7FFF) > 0x7C00
+
+
 def test_ragged_list_equals_flat_tensor(O, L, host, B, torch_gpu):
     """4,096 tensors of 128..65,536 elements in one launch against one flat tensor with the same
     values: identical bits, and both equal to the oracle."""
