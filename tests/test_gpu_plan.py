@@ -5,7 +5,7 @@ import os
 import numpy as np
 import pytest
 
-from util import HYPER, bits, check_state
+from util import HYPER, bits, check_state, read_device
 
 pytestmark = pytest.mark.gpu
 
@@ -153,6 +153,33 @@ def test_grad_norm_and_clip(O, L, host, B, torch_gpu, chunk):
     oracle_step(O, L, specs, hs, 1, dict(HYPER, lr=1e-3))
     assert compare(stores[0], hs, "unfused") == 0
     assert compare(stores[1], hs, "fused") == 0
+
+
+@pytest.mark.parametrize("chunk", [512, 1024, 2048, 4096, 8192, 65536])
+def test_norm_partials_on_wide_range_gradients(O, L, host, B, torch_gpu, chunk):
+    """Gradients that are uniformly random finite FP16 bit patterns (magnitudes from 6e-8 to 65504, so FP32
+    accumulators round at every addition) and FP32 gradients spread over forty binades: every per-chunk partial
+    and the total equal the restated reduction order bit for bit, for each width of the norm workgroup."""
+    torch = torch_gpu
+    rng = np.random.default_rng(chunk)
+    n16, n32 = 300_007, 70_001
+    h = rng.integers(0, 1 << 16, n16, dtype=np.uint32).astype(np.uint16)
+    h[(h & 0x7C00) == 0x7C00] &= 0x83FF                      # infinities and NaNs become subnormals
+    f = (rng.standard_normal(n32) * np.exp2(rng.integers(-20, 20, n32))).astype(np.float32)
+    g16 = torch.from_numpy(h.view(np.int16)).to("cuda:0").view(torch.float16)
+    g32 = torch.from_numpy(f).to("cuda:0")
+    descs = [B.TensorDesc(None, g16.data_ptr(), None, None, None, n16, B.DTYPE_F16, B.TENSOR_GRAD_ONLY),
+             B.TensorDesc(None, g32.data_ptr(), None, None, None, n32, B.DTYPE_F32, B.TENSOR_GRAD_ONLY)]
+    plan = B.Plan(descs, chunk)
+    plan.grad_norm(1.0)
+    norm, scale, sum_sq = plan.norm_read()
+    mirror, parts = O.sumsq_mirror([h, f], chunk)
+    assert parts.size == plan.num_chunks
+    dev_parts = read_device(plan.partials_ptr, 8 * plan.num_chunks).view(np.float64)
+    assert np.array_equal(dev_parts.view(np.uint64), parts.view(np.uint64)), "partials differ"
+    assert sum_sq == mirror
+    truth = float((O.h2f(h).astype(np.float64) ** 2).sum() + (f.astype(np.float64) ** 2).sum())
+    assert abs(sum_sq - truth) <= 1e-5 * truth
 
 
 def test_norm_below_threshold_touches_nothing(O, L, host, torch_gpu):

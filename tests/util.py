@@ -38,3 +38,16 @@ def check_state(got_p, got_m, got_v, exp_p, exp_m, exp_v, what=""):
         assert rel_err(got_p, exp_p).max() <= 1e-6, what + " p"
     return int((got_p != exp_p).sum() + (got_m.view(np.uint32) != exp_m.view(np.uint32)).sum()
                + (got_v.view(np.uint32) != exp_v.view(np.uint32)).sum())
+
+
+def read_device(ptr, nbytes):
+    """Bytes at a raw device address, copied with the HIP runtime that the process already has loaded."""
+    import ctypes as C
+    path = next(line.split()[-1] for line in open("/proc/self/maps") if "libamdhip64" in line)
+    hip = C.CDLL(path)
+    hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
+    hip.hipMemcpy.restype = C.c_int
+    buf = np.empty(nbytes, np.uint8)
+    rc = hip.hipMemcpy(buf.ctypes.data, ptr, nbytes, 2)          # 2 = device to host; waits for earlier work
+    assert rc == 0, "hipMemcpy failed: %d" % rc
+    return buf
