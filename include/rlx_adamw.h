@@ -62,6 +62,16 @@ int rlx_adamw_fp32(float* w, const float* grad, float* m, float* v, int64_t n,
 /* Replaces fp16_to_fp32 (include/training/optimizer.h:46-57): dst[i] = (float)src[i]. */
 int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream);
 
+/*
+ * Zero fill of nbytes at dst, any alignment, as kernels: replaces the two cudaMemsetAsync of
+ * qwen3_gradients_zero (src/model/qwen3.cu:1109-1112) and the memset of the frozen embedding's
+ * gradients (include/training/trainer.h:271-277) where the caller records its step into a HIP
+ * graph (memset nodes are avoided there) or wants the same stream-ordered call either way.
+ * nbytes <= 0 is a no-op.  (rlx_plan_adamw with RLX_STEP_ZERO_GRADS makes it unnecessary for
+ * the gradient pools.)
+ */
+int rlx_clear(void* dst, int64_t nbytes, void* stream);
+
 /* ------------------------------------------------------------------------------------
  * Multi-tensor plan: a whole model's tensors in one launch.
  * ---------------------------------------------------------------------------------- */

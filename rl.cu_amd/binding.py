@@ -45,6 +45,7 @@ SIGNATURES = {
     "rlx_adamw_fp16": ([_VP, _VP, _VP, _VP, _VP, _I64] + _HYPER + [_VP], _INT),
     "rlx_adamw_fp32": ([_VP, _VP, _VP, _VP, _I64] + _HYPER + [_VP], _INT),
     "rlx_fp16_to_fp32": ([_VP, _VP, _I64, _VP], _INT),
+    "rlx_clear": ([_VP, _I64, _VP], _INT),
     "rlx_plan_create": ([C.POINTER(TensorDesc), _I64, _I64, C.POINTER(_VP)], _INT),
     "rlx_plan_layout": ([C.POINTER(TensorDesc), _I64, _I64, C.POINTER(_I64), C.POINTER(_I64), C.POINTER(_I64)], _INT),
     "rlx_plan_destroy": ([_VP], _INT),
@@ -141,6 +142,10 @@ def fill_f16(dst, n, seed, mean, std, first=0, flags=0, row_len=0, zero_rows_bel
 def fill_f32(dst, n, seed, mean, std, first=0, flags=0, row_len=0, zero_rows_below=0, stream=0):
     check(load().rlx_fill_f32(dst, n, seed, first, mean, std, flags, row_len, zero_rows_below, stream),
           "rlx_fill_f32")
+
+
+def clear(dst, nbytes, stream=0):
+    check(load().rlx_clear(dst, nbytes, stream), "rlx_clear")
 
 
 def plan_layout(descs, chunk_elems=0):

@@ -533,6 +533,22 @@ __global__ __launch_bounds__(256) void fp16_to_fp32_kernel(float* __restrict__ d
         dst[i] = h2f(src[i]);
 }
 
+// Zero fill as a kernel (a memset node recorded into a HIP graph is not reliable on every
+// runtime; a kernel is).  One workgroup of 256 lanes per 4 KiB: one 128-bit store per lane.
+// `body` points at a 16-byte boundary; the few bytes before and after it are written by the host
+// launcher's second, byte-wise launch.
+__global__ __launch_bounds__(256) void clear_body_kernel(u32x4* __restrict__ body, int64_t n_vec) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n_vec) st_stream<1>(body + i, u32x4{0u, 0u, 0u, 0u});
+}
+
+__global__ __launch_bounds__(64) void clear_edges_kernel(uint8_t* __restrict__ head, int n_head,
+                                                         uint8_t* __restrict__ tail, int n_tail) {
+    const int t = threadIdx.x;
+    if (t < n_head) head[t] = 0;
+    if (t < n_tail) tail[t] = 0;
+}
+
 // ---------------------------------------------------------------------------------------
 // Seeded synthetic inputs: integer hash -> sum of eight 16-bit uniforms -> one FP32
 // multiply and one FP32 add, so that a host restatement gives the same bits without libm.
@@ -777,7 +793,7 @@ const char* rlx_status_string(int status) {
 
 const char* rlx_last_hip_error(void) { return g_hip_error; }
 
-int rlx_version(void) { return 103; }
+int rlx_version(void) { return 104; }
 
 int rlx_adamw_fp16(float* master_w, uint16_t* model_w, const uint16_t* grad, float* m, float* v, int64_t n,
                    float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -800,6 +816,27 @@ int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream) {
     int64_t grid = (n + 255) / 256;
     if (grid > 65536) grid = 65536;
     fp16_to_fp32_kernel<<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(dst, src, n);
+    RLX_HIP(hipGetLastError());
+    return RLX_OK;
+}
+
+int rlx_clear(void* dst, int64_t nbytes, void* stream) {
+    if (nbytes <= 0) return RLX_OK;
+    if (!dst) return RLX_ERR_INVALID_ARG;
+    hipStream_t s = (hipStream_t)stream;
+    uint8_t* b = (uint8_t*)dst;
+    int64_t n_head = (int64_t)((16 - ((uintptr_t)b & 15)) & 15);
+    if (n_head > nbytes) n_head = nbytes;
+    const int64_t n_vec = (nbytes - n_head) / 16;
+    const int64_t n_tail = nbytes - n_head - n_vec * 16;
+    u32x4* body = (u32x4*)(b + n_head);
+    const int64_t per_launch = kMaxTilesPerLaunch * 256;         // vectors per launch
+    for (int64_t first = 0; first < n_vec; first += per_launch) {
+        const int64_t here = n_vec - first < per_launch ? n_vec - first : per_launch;
+        clear_body_kernel<<<dim3((unsigned)((here + 255) / 256)), dim3(256), 0, s>>>(body + first, here);
+    }
+    if (n_head || n_tail)
+        clear_edges_kernel<<<dim3(1), dim3(64), 0, s>>>(b, (int)n_head, b + n_head + n_vec * 16, (int)n_tail);
     RLX_HIP(hipGetLastError());
     return RLX_OK;
 }

@@ -72,6 +72,53 @@ struct GradPools {
     size_t float_pool_bytes = 0;
 };
 
+// Allocation, clearing and release of the gradient pools: the roles of qwen3_gradients_alloc, _zero and
+// _free (src/model/qwen3.cu:1016-1112).  workspace_floats is the tail behind the norm gradients
+// (max_T * num_attention_heads floats in the reference).  The pools come back cleared.
+inline void grad_pools_zero(GradPools* g, hipStream_t stream = 0) {
+    RLX_CHECK(rlx_clear(g->half_pool, (int64_t)g->half_pool_bytes, (void*)stream));
+    RLX_CHECK(rlx_clear(g->float_pool, (int64_t)g->float_pool_bytes, (void*)stream));
+}
+
+inline GradPools grad_pools_alloc(const ParamPools& pools, size_t workspace_floats) {
+    GradPools g;
+    g.half_pool_bytes = pools.fp16_pool_elems * sizeof(half);
+    g.float_pool_bytes = (pools.fp32_pool_elems + workspace_floats) * sizeof(float);
+    if (g.half_pool_bytes) HIP_CHECK(hipMalloc((void**)&g.half_pool, g.half_pool_bytes));
+    if (g.float_pool_bytes) HIP_CHECK(hipMalloc((void**)&g.float_pool, g.float_pool_bytes));
+    grad_pools_zero(&g);
+    HIP_CHECK(hipDeviceSynchronize());
+    return g;
+}
+
+inline void grad_pools_free(GradPools* g) {
+    if (g->half_pool) (void)hipFree(g->half_pool);
+    if (g->float_pool) (void)hipFree(g->float_pool);
+    *g = GradPools();
+}
+
+// Where one tensor's gradient lies in the pools: what the dW_* pointer arrays of Qwen3Gradients hold
+// (include/model/qwen3.h:190-218).  proj: 0=q 1=k 2=v 3=o 4=gate 5=up 6=down; norm: 0=input 1=q 2=k
+// 3=post_attn.  They need the per-layer structure in ParamPools.
+inline size_t pool_offset(const size_t* sizes, int count, int layer, int which) {
+    size_t per = 0, off = 0;
+    for (int i = 0; i < count; i++) { per += sizes[i]; if (i < which) off += sizes[i]; }
+    return (size_t)layer * per + off;
+}
+inline half* grad_proj(const GradPools& g, const ParamPools& p, int layer, int proj) {
+    assert(layer >= 0 && layer < p.num_layers && proj >= 0 && proj < 7);
+    return g.half_pool + pool_offset(p.proj_sizes, 7, layer, proj);
+}
+inline half* grad_embed(const GradPools& g, const ParamPools& p) { return g.half_pool + p.proj_elems; }
+inline float* grad_norm_weight(const GradPools& g, const ParamPools& p, int layer, int norm) {
+    assert(layer >= 0 && layer < p.num_layers && norm >= 0 && norm < 4);
+    return g.float_pool + pool_offset(p.norm_sizes, 4, layer, norm);
+}
+inline float* grad_final_norm(const GradPools& g, const ParamPools& p) {
+    return g.float_pool + pool_offset(p.norm_sizes, 4, p.num_layers, 0);
+}
+inline float* grad_workspace(const GradPools& g, const ParamPools& p) { return g.float_pool + p.fp32_pool_elems; }
+
 class AdamWOptimizer {
 public:
     // Hyper-parameters (public, as in the reference)
@@ -266,15 +313,11 @@ private:
 
     size_t fp16_offset(int layer, int proj) const {
         assert(pools_.num_layers > 0 && layer >= 0 && layer < pools_.num_layers && proj >= 0 && proj < 7);
-        size_t per = 0, off = 0;
-        for (int i = 0; i < 7; i++) { per += pools_.proj_sizes[i]; if (i < proj) off += pools_.proj_sizes[i]; }
-        return (size_t)layer * per + off;
+        return pool_offset(pools_.proj_sizes, 7, layer, proj);
     }
     size_t fp32_offset(int layer, int norm) const {
         assert(pools_.num_layers > 0 && layer >= 0 && layer <= pools_.num_layers && norm >= 0 && norm < 4);
-        size_t per = 0, off = 0;
-        for (int i = 0; i < 4; i++) { per += pools_.norm_sizes[i]; if (i < norm) off += pools_.norm_sizes[i]; }
-        return (size_t)layer * per + off;
+        return pool_offset(pools_.norm_sizes, 4, layer, norm);
     }
 
     struct Section { std::string name; float* dev; size_t n; };

@@ -41,9 +41,8 @@ public:
         if (config_.freeze_embed && !config_.freeze_in_plan && embed_elems) {
             const size_t half_elems = grads->half_pool_bytes / sizeof(half);
             half* embed_grad = grads->half_pool + (half_elems - embed_elems);
-            // zeros through a fill kernel (0 + 0 * z), which unlike a memset node is safe to capture
-            RLX_CHECK(rlx_fill_f16(reinterpret_cast<uint16_t*>(embed_grad), (int64_t)embed_elems, 0, 0, 0.0f, 0.0f, 0,
-                                   0, 0, (void*)stream));
+            // cleared by a kernel, which unlike a memset node is safe to record into a HIP graph
+            RLX_CHECK(rlx_clear(embed_grad, (int64_t)(embed_elems * sizeof(half)), (void*)stream));
         }
         float grad_norm = 0.0f;
         const bool clip = config_.max_grad_norm > 0.0f;

@@ -348,6 +348,60 @@ static void test_train_loop() {
     else FAIL(name, "lines=%d shape=%d", lines, shape);
 }
 
+// 10. Gradient pools: sizes and pointer partition of qwen3_gradients_alloc (src/model/qwen3.cu:1016-1085),
+//     cleared on allocation and by grad_pools_zero; rlx_clear at odd addresses leaves its neighbours alone
+static void test_grad_pools() {
+    const char* name = "gradient pools: alloc, partition, zero";
+    // Qwen3-0.6B dimensions with 2 layers and a small vocabulary
+    const int L = 2, H = 1024, QD = 2048, KVD = 1024, I = 3072, HD = 128, V = 1000, max_T = 64, heads = 16;
+    ParamPools pools = ParamPools::for_qwen3(L, H, QD, KVD, I, HD, V);
+    GradPools g = grad_pools_alloc(pools, (size_t)max_T * heads);
+    const size_t per16 = (size_t)QD * H + 2 * (size_t)KVD * H + (size_t)H * QD + 3 * (size_t)I * H;
+    const size_t per32 = 2 * (size_t)H + 2 * HD;
+    bool ok = g.half_pool_bytes == (per16 * L + (size_t)V * H) * 2 &&
+              g.float_pool_bytes == (per32 * L + H + (size_t)max_T * heads) * 4;
+    ok = ok && grad_proj(g, pools, 0, 0) == g.half_pool && grad_proj(g, pools, 0, 1) == g.half_pool + (size_t)QD * H &&
+         grad_proj(g, pools, 1, 0) == g.half_pool + per16 &&
+         grad_proj(g, pools, 1, 6) == g.half_pool + 2 * per16 - (size_t)H * I &&
+         grad_embed(g, pools) == g.half_pool + per16 * L &&
+         grad_norm_weight(g, pools, 0, 1) == g.float_pool + H && grad_norm_weight(g, pools, 1, 3) == g.float_pool + per32 + H + 2 * HD &&
+         grad_final_norm(g, pools) == g.float_pool + per32 * L && grad_workspace(g, pools) == g.float_pool + per32 * L + H;
+    std::vector<uint16_t> h16 = d2h((const uint16_t*)g.half_pool, g.half_pool_bytes / 2);
+    std::vector<float> h32 = d2h((const float*)g.float_pool, g.float_pool_bytes / 4);
+    size_t nonzero = 0;
+    for (uint16_t x : h16) nonzero += x != 0;
+    for (float x : h32) nonzero += x != 0.0f;
+    // dirty both pools, clear them again
+    RLX_CHECK(rlx_fill_f16((uint16_t*)g.half_pool, g.half_pool_bytes / 2, 9, 0, 1.0f, 0.1f, 0, 0, 0, nullptr));
+    RLX_CHECK(rlx_fill_f32(g.float_pool, g.float_pool_bytes / 4, 9, 0, 1.0f, 0.1f, 0, 0, 0, nullptr));
+    grad_pools_zero(&g);
+    HIP_CHECK(hipDeviceSynchronize());
+    h16 = d2h((const uint16_t*)g.half_pool, g.half_pool_bytes / 2);
+    h32 = d2h((const float*)g.float_pool, g.float_pool_bytes / 4);
+    for (uint16_t x : h16) nonzero += x != 0;
+    for (float x : h32) nonzero += x != 0.0f;
+    // rlx_clear on ranges that start and end at odd byte addresses
+    size_t wrong = 0;
+    const size_t span = 1000;
+    unsigned char* buf = nullptr;
+    HIP_CHECK(hipMalloc((void**)&buf, span));
+    const int cases[][2] = {{0, 1000}, {1, 1}, {3, 13}, {15, 17}, {16, 16}, {7, 990}, {33, 0}, {5, 40}};
+    for (const auto& c : cases) {
+        HIP_CHECK(hipMemset(buf, 0xAB, span));
+        RLX_CHECK(rlx_clear(buf + c[0], c[1], nullptr));
+        HIP_CHECK(hipDeviceSynchronize());
+        std::vector<unsigned char> h = d2h((const unsigned char*)buf, span);
+        for (size_t i = 0; i < span; i++) {
+            const bool inside = i >= (size_t)c[0] && i < (size_t)(c[0] + c[1]);
+            wrong += h[i] != (inside ? 0x00 : 0xAB);
+        }
+    }
+    (void)hipFree(buf);
+    grad_pools_free(&g);
+    ok = ok && g.half_pool == nullptr && g.float_pool_bytes == 0;
+    if (ok && nonzero == 0 && wrong == 0) PASS(name); else FAIL(name, "ok=%d nonzero=%zu wrong=%zu", ok, nonzero, wrong);
+}
+
 int main() {
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
@@ -364,6 +418,7 @@ int main() {
     test_frozen_and_zeroing();
     test_checkpoint();
     test_train_loop();
+    test_grad_pools();
     printf("=== %s (%d failure%s) ===\n", g_fails ? "FAILED" : "ALL PASSED", g_fails, g_fails == 1 ? "" : "s");
     return g_fails;
 }

@@ -260,3 +260,23 @@ def test_fp32_update_on_random_bit_patterns(O, B, host, torch_gpu):
         assert not bad.any(), "%s: %d differ, first at %d" % (what, int(bad.sum()), int(np.argmax(bad)))
         finite += int(np.isfinite(exp).sum())
     assert finite > n        # most results are numbers, not NaN
+
+
+def test_clear_any_alignment_and_size(B, torch_gpu):
+    """rlx_clear writes zeros to exactly the requested bytes: odd starts, odd lengths, and a range of more
+    than 2 GiB; the bytes either side keep their pattern."""
+    torch = torch_gpu
+    span = 70_000
+    for start, nbytes in [(0, span), (1, 1), (3, 13), (15, 17), (16, 4096), (5, 65_000), (129, 0), (31, 33)]:
+        buf = torch.full((span,), 0xAB, dtype=torch.uint8, device="cuda:0")
+        B.clear(buf.data_ptr() + start, nbytes)
+        torch.cuda.synchronize()
+        h = buf.cpu().numpy()
+        exp = np.full(span, 0xAB, np.uint8)
+        exp[start:start + nbytes] = 0
+        assert np.array_equal(h, exp), (start, nbytes)
+    big = torch.full(((1 << 31) + 4099,), 0x5A, dtype=torch.uint8, device="cuda:0")
+    B.clear(big.data_ptr() + 3, (1 << 31) + 4090)
+    torch.cuda.synchronize()
+    assert int(big[:3].sum()) == 3 * 0x5A and int(big[-6:].sum()) == 6 * 0x5A
+    assert int(big[3:-6].max()) == 0
