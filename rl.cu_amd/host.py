@@ -152,6 +152,12 @@ class ParamStore:
                 fn = B.fill_f32
             fn(t.data_ptr(), s.n, ts, mean, std, 0, flags, row_len, zt, st)
 
+    def zero_grads(self, stream=None):
+        """Clears both gradient pools (qwen3_gradients_zero, src/model/qwen3.cu:1109-1112)."""
+        st = _stream() if stream is None else stream
+        B.clear(self.g16.data_ptr(), self.g16.numel() * 2, st)
+        B.clear(self.g32.data_ptr(), self.g32.numel() * 4, st)
+
     def init_master(self):
         """master = (float)param for FP16 tensors (optimizer.h:242)."""
         st = _stream()

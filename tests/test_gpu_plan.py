@@ -358,10 +358,12 @@ def test_zero_grads_in_the_update_and_frozen_embedding(O, L, host, B, torch_gpu)
     torch.cuda.synchronize()
     hs = host_copy(st_a)
     for step in range(1, 4):
+        st_a.zero_grads()                                        # qwen3_gradients_zero, then "backward":
+        assert not st_a.g16.any().item() and not st_a.g32.any().item()
         for st, tail in ((st_a, tails[0]), (st_b, tails[1])):
             st.fill("g", 50 + step, 0.0, 5e-3)
             B.fill_f32(tail.data_ptr(), 555, 60 + step, 0.0, 0.1)
-        st_a.grad(emb).zero_()                                   # the reference's freeze_embed memset
+        B.clear(st_a.grad(emb).data_ptr(), ref_specs[emb].n * 2)  # the reference's freeze_embed memset
         torch.cuda.synchronize()
         for i, h in enumerate(hs):
             h["g"] = bits(st_a.grad(i))
