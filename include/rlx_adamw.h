@@ -63,6 +63,13 @@ int rlx_adamw_fp32(float* w, const float* grad, float* m, float* v, int64_t n,
 int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream);
 
 /*
+ * x[i] *= scale over a plain FP32 buffer: replaces scale_grad_kernel (include/training/trainer.h:93-99),
+ * with which training_step divides each micro-batch's loss gradient by grad_accum_steps before the
+ * backward pass adds it into the gradient pools (trainer.h:261-263).
+ */
+int rlx_scale_f32(float* x, float scale, int64_t n, void* stream);
+
+/*
  * Zero fill of nbytes at dst, any alignment, as kernels: replaces the two cudaMemsetAsync of
  * qwen3_gradients_zero (src/model/qwen3.cu:1109-1112) and the memset of the frozen embedding's
  * gradients (include/training/trainer.h:271-277) where the caller records its step into a HIP

@@ -46,6 +46,7 @@ SIGNATURES = {
     "rlx_adamw_fp32": ([_VP, _VP, _VP, _VP, _I64] + _HYPER + [_VP], _INT),
     "rlx_fp16_to_fp32": ([_VP, _VP, _I64, _VP], _INT),
     "rlx_clear": ([_VP, _I64, _VP], _INT),
+    "rlx_scale_f32": ([_VP, _F, _I64, _VP], _INT),
     "rlx_plan_create": ([C.POINTER(TensorDesc), _I64, _I64, C.POINTER(_VP)], _INT),
     "rlx_plan_layout": ([C.POINTER(TensorDesc), _I64, _I64, C.POINTER(_I64), C.POINTER(_I64), C.POINTER(_I64)], _INT),
     "rlx_plan_destroy": ([_VP], _INT),
@@ -146,6 +147,10 @@ def fill_f32(dst, n, seed, mean, std, first=0, flags=0, row_len=0, zero_rows_bel
 
 def clear(dst, nbytes, stream=0):
     check(load().rlx_clear(dst, nbytes, stream), "rlx_clear")
+
+
+def scale_f32(x, scale, n, stream=0):
+    check(load().rlx_scale_f32(x, scale, n, stream), "rlx_scale_f32")
 
 
 def plan_layout(descs, chunk_elems=0):

@@ -526,6 +526,21 @@ __global__ __launch_bounds__(BLOCK) void scale_group_kernel(
     }
 }
 
+// x[i] *= scale for a plain FP32 buffer (the per-micro-batch loss-gradient scale, trainer.h:96-99).
+// The buffer is small (one value per token); 128-bit accesses when it is 16-byte aligned.
+__global__ __launch_bounds__(256) void scale_f32_kernel(float* __restrict__ x, float scale, int64_t n, int vec_ok) {
+    const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n) return;
+    if (vec_ok && i + 4 <= n) {
+        f32x4 v = ldg<false>((const f32x4*)(x + i));
+#pragma unroll
+        for (int k = 0; k < 4; k++) v[k] = v[k] * scale;
+        stg<false>((f32x4*)(x + i), v);
+    } else {
+        for (int64_t j = i; j < i + 4 && j < n; j++) x[j] = x[j] * scale;
+    }
+}
+
 __global__ __launch_bounds__(256) void fp16_to_fp32_kernel(float* __restrict__ dst,
                                                            const uint16_t* __restrict__ src, int64_t n)
 {
@@ -793,7 +808,7 @@ const char* rlx_status_string(int status) {
 
 const char* rlx_last_hip_error(void) { return g_hip_error; }
 
-int rlx_version(void) { return 104; }
+int rlx_version(void) { return 105; }
 
 int rlx_adamw_fp16(float* master_w, uint16_t* model_w, const uint16_t* grad, float* m, float* v, int64_t n,
                    float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -816,6 +831,21 @@ int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream) {
     int64_t grid = (n + 255) / 256;
     if (grid > 65536) grid = 65536;
     fp16_to_fp32_kernel<<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(dst, src, n);
+    RLX_HIP(hipGetLastError());
+    return RLX_OK;
+}
+
+int rlx_scale_f32(float* x, float scale, int64_t n, void* stream) {
+    if (n <= 0) return RLX_OK;
+    if (!x) return RLX_ERR_INVALID_ARG;
+    if (!is_aligned(x, 4)) return RLX_ERR_MISALIGNED;
+    const int64_t lanes = (n + 3) / 4;
+    const int64_t per_launch = kMaxTilesPerLaunch * 256;         // lanes per launch
+    for (int64_t first = 0; first < lanes; first += per_launch) {
+        const int64_t here = lanes - first < per_launch ? lanes - first : per_launch;
+        scale_f32_kernel<<<dim3((unsigned)((here + 255) / 256)), dim3(256), 0, (hipStream_t)stream>>>(
+            x + first * 4, scale, n - first * 4, is_aligned(x, 16) ? 1 : 0);
+    }
     RLX_HIP(hipGetLastError());
     return RLX_OK;
 }

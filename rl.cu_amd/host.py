@@ -291,6 +291,32 @@ def training_step(optimizer, max_grad_norm, fused_clip=False, zero_grads=False):
     return grad_norm
 
 
+def accumulation_step(optimizer, micro_batch, grad_accum_steps, max_grad_norm, loss_grad=None, fused_clip=False,
+                      freeze=None, stream=None):
+    """Trainer::training_step around the optimizer (include/training/trainer.h:231-289): clear the gradient
+    pools; for each of grad_accum_steps micro-batches call micro_batch(k, scale_loss_grad) -> loss, which
+    stands for forward, compute_loss and backward: it fills `loss_grad` (a torch FP32 tensor), calls
+    scale_loss_grad() where the reference launches scale_grad_kernel (between compute_loss and backward,
+    trainer.h:261-263) and adds its gradients into the pools; then clear the gradients of the tensor views
+    in `freeze` (freeze_embed), clip, step.  Returns (mean loss, pre-clip norm)."""
+    import numpy as np
+    st = _stream() if stream is None else stream
+    optimizer.store.zero_grads(st)
+    scale = float(np.float32(1.0) / np.float32(grad_accum_steps))
+
+    def scale_loss_grad():
+        if loss_grad is not None:
+            B.scale_f32(loss_grad.data_ptr(), scale, loss_grad.numel(), st)
+
+    accum = 0.0
+    for k in range(grad_accum_steps):
+        accum += micro_batch(k, scale_loss_grad)
+    for t in (freeze or ()):
+        B.clear(t.data_ptr(), t.numel() * t.element_size(), st)
+    grad_norm = training_step(optimizer, max_grad_norm, fused_clip=fused_clip)
+    return accum / grad_accum_steps, grad_norm
+
+
 class Logger:
     """JSON-lines metrics logger with the reference's interface (include/training/logger.h:27-128):
     log() accumulates, commit() writes the window's means as one object with a "step" key, appends to

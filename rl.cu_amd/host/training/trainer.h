@@ -52,6 +52,26 @@ public:
         return grad_norm;
     }
 
+    // Trainer::training_step around the optimizer (trainer.h:231-289): clear the gradient pools, run
+    // grad_accum_steps micro-batches, then apply().  micro_batch(k, scale_loss_grad) stands for forward,
+    // compute_loss and backward of micro-batch k and returns its loss; it calls scale_loss_grad(d_loss_grad, n)
+    // where the reference launches scale_grad_kernel (trainer.h:261-263), before its backward pass adds
+    // into the pools.  Returns the mean loss; the pre-clip norm is last_grad_norm().
+    using ScaleLossGrad = std::function<void(float*, size_t)>;
+    float training_step(GradPools* grads, int grad_accum_steps,
+                        const std::function<float(int, const ScaleLossGrad&)>& micro_batch, size_t embed_elems = 0,
+                        hipStream_t stream = 0) {
+        const float scale = 1.0f / (float)grad_accum_steps;
+        grad_pools_zero(grads, stream);
+        const ScaleLossGrad scale_loss_grad = [scale, stream](float* d_loss_grad, size_t n) {
+            RLX_CHECK(rlx_scale_f32(d_loss_grad, scale, (int64_t)n, (void*)stream));
+        };
+        float accum_loss = 0.0f;
+        for (int acc = 0; acc < grad_accum_steps; acc++) accum_loss += micro_batch(acc, scale_loss_grad);
+        apply(grads, embed_elems, stream);
+        return accum_loss / (float)grad_accum_steps;
+    }
+
     float last_grad_norm() const { return last_grad_norm_; }
 
 private:

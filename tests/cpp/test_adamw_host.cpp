@@ -402,6 +402,51 @@ static void test_grad_pools() {
     if (ok && nonzero == 0 && wrong == 0) PASS(name); else FAIL(name, "ok=%d nonzero=%zu wrong=%zu", ok, nonzero, wrong);
 }
 
+// 11. training_step with gradient accumulation: pools cleared first, loss gradient scaled by 1/acc_steps,
+//     then clip + step; equals doing the same by hand
+static void test_accumulation() {
+    const char* name = "training_step: clear, scaled micro-batches, clip, step";
+    Fixture fa(5e-3f), fb(5e-3f);
+    AdamWOptimizer oa(fa.pools, 1e-3f), ob(fb.pools, 1e-3f);
+    OptimStepConfig cfg;
+    cfg.max_grad_norm = 0.5f;
+    cfg.fused_clip = true;
+    OptimStep sa(&oa, cfg), sb(&ob, cfg);
+    const int acc = 4;
+    const size_t T = 50;
+    float* lg = nullptr;
+    HIP_CHECK(hipMalloc((void**)&lg, T * 4));
+    std::vector<float> seen;      // loss_grad[0] after scaling, per micro-batch
+    // stand-in backward: the last micro-batch writes seeded gradients (so the pools' final content is known)
+    auto micro = [&](int k, const OptimStep::ScaleLossGrad& scale_loss_grad) {
+        RLX_CHECK(rlx_fill_f32(lg, T, 40 + k, 0, 3.0f, 0.0f, 0, 0, 0, nullptr));
+        scale_loss_grad(lg, T);
+        seen.push_back(d2h((const float*)lg, 1)[0]);
+        if (k == 0) {             // the pools must have been cleared before the first micro-batch
+            std::vector<uint16_t> h = d2h((const uint16_t*)fa.g16, fa.n16);
+            size_t nz = 0;
+            for (uint16_t x : h) nz += x != 0;
+            if (nz) seen.push_back(-1.0f);
+        }
+        if (k == acc - 1) {
+            RLX_CHECK(rlx_fill_f16((uint16_t*)fa.g16, fa.n16, 2, 0, 0.0f, 5e-3f, 0, 0, 0, nullptr));
+            RLX_CHECK(rlx_fill_f32(fa.g32, fa.n32 + fa.tail, 4, 0, 0.0f, 5e-3f, 0, 0, 0, nullptr));
+        }
+        return (float)(k + 1);
+    };
+    const float loss = sa.training_step(&fa.grads, acc, micro);
+    const float nb = sb.apply(&fb.grads);           // fb still holds the same seeded gradients
+    HIP_CHECK(hipDeviceSynchronize());
+    bool scaled = seen.size() == (size_t)acc;
+    for (float x : seen) scaled = scaled && x == 3.0f * (1.0f / (float)acc);
+    std::vector<uint16_t> wa = d2h((const uint16_t*)fa.w16, fa.n16), wb = d2h((const uint16_t*)fb.w16, fb.n16);
+    size_t diff = 0;
+    for (size_t i = 0; i < fa.n16; i++) diff += wa[i] != wb[i];
+    (void)hipFree(lg);
+    if (scaled && loss == 2.5f && sa.last_grad_norm() == nb && nb > 0.5f && diff == 0) PASS(name);
+    else FAIL(name, "scaled=%d loss=%f na=%f nb=%f diff=%zu", scaled, loss, sa.last_grad_norm(), nb, diff);
+}
+
 int main() {
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
@@ -419,6 +464,7 @@ int main() {
     test_checkpoint();
     test_train_loop();
     test_grad_pools();
+    test_accumulation();
     printf("=== %s (%d failure%s) ===\n", g_fails ? "FAILED" : "ALL PASSED", g_fails, g_fails == 1 ? "" : "s");
     return g_fails;
 }

@@ -280,3 +280,19 @@ def test_clear_any_alignment_and_size(B, torch_gpu):
     torch.cuda.synchronize()
     assert int(big[:3].sum()) == 3 * 0x5A and int(big[-6:].sum()) == 6 * 0x5A
     assert int(big[3:-6].max()) == 0
+
+
+@pytest.mark.parametrize("n,offset", [(1, 0), (3, 0), (4, 1), (4096, 0), (4097, 3), (1_000_003, 2)])
+def test_scale_f32_equals_the_oracle(O, B, torch_gpu, n, offset):
+    """The loss-gradient scale by 1/grad_accum_steps (include/training/trainer.h:96-99,261-263): one FP32
+    multiply per element, any start alignment; the elements either side are untouched."""
+    torch = torch_gpu
+    buf = torch.empty(n + offset + 5, dtype=torch.float32, device="cuda:0")
+    B.fill_f32(buf.data_ptr(), n + offset + 5, 77, 0.0, 3.0)
+    torch.cuda.synchronize()
+    h = bits(buf)
+    scale = float(np.float32(1.0) / np.float32(3.0))
+    B.scale_f32(buf.data_ptr() + 4 * offset, scale, n)
+    O.scale_float(h[offset:offset + n], scale)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(buf).view(np.uint32), h.view(np.uint32))

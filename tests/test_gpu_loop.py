@@ -217,3 +217,69 @@ def test_two_host_threads_with_their_own_plans_and_streams(O, L, host, B, torch_
         for i in range(2):
             assert np.array_equal(bits(stores[k].param(i)), hs[i]["p"])
             assert np.array_equal(bits(stores[k].state(i, "v")), hs[i]["v"])
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_accumulation_step_follows_the_reference_order(O, L, host, B, torch_gpu, fused):
+    """training_step of the reference (include/training/trainer.h:231-289) with three micro-batches: clear
+    the pools, scale each micro-batch's loss gradient by 1/3 before its backward pass adds into the pools,
+    clear the frozen embedding's gradients, clip, step.  The backward pass here is a stand-in made of
+    element-wise operations only (so that host and device agree exactly); everything else is the library,
+    checked against numpy + the oracle in the same order."""
+    import numpy as np
+    from util import HYPER, bits
+    from test_gpu_plan import compare, host_copy, oracle_step
+    torch = torch_gpu
+    specs, st, opt = make(L, host, master=False)
+    emb = [i for i, s in enumerate(specs) if s.name == "embed_tokens"][0]
+    acc, T = 3, 37
+    loss_grad = torch.empty(T, dtype=torch.float32, device="cuda:0")
+    st.fill("g", 999, 0.0, 1.0)                       # stale gradients that the step must clear first
+    torch.cuda.synchronize()
+    hs = host_copy(st)
+    for h in hs:
+        h["g"][...] = 0
+    scale = np.float32(1.0) / np.float32(acc)
+    base16 = [torch.empty_like(st.g16), None]
+    base32 = torch.empty_like(st.g32)
+
+    def micro_batch(k, scale_loss_grad):
+        B.fill_f32(loss_grad.data_ptr(), T, 500 + k, 2.0, 0.5)          # "compute_loss"
+        lg_h = O.fill_f32(T, 500 + k, 2.0, 0.5)
+        scale_loss_grad()
+        lg_h = lg_h * scale
+        # "backward": pools += seeded pattern * loss_grad[0], element-wise
+        B.fill_f16(base16[0].data_ptr(), base16[0].numel(), 600 + k, 0.0, 2e-3)
+        B.fill_f32(base32.data_ptr(), base32.numel(), 700 + k, 0.0, 2e-3)
+        f = loss_grad[0]
+        st.g16.add_((base16[0].float() * f).half())
+        st.g32.add_(base32 * f)
+        b16 = O.h2f(O.fill_f16(base16[0].numel(), 600 + k, 0.0, 2e-3))
+        b32 = O.fill_f32(base32.numel(), 700 + k, 0.0, 2e-3)
+        for i, s in enumerate(specs):
+            lo = st.off_pg[i]
+            if s.dtype == L.DTYPE_F16:
+                add = (b16[lo:lo + s.n] * lg_h[0]).astype(np.float16)
+                cur = hs[i]["g"].view(np.float16)
+                hs[i]["g"] = (cur.astype(np.float32) + add.astype(np.float32)).astype(np.float16).view(np.uint16)
+            else:
+                hs[i]["g"] = (hs[i]["g"] + b32[lo:lo + s.n] * lg_h[0]).astype(np.float32)
+        return float(k + 1)
+
+    loss, norm = host.accumulation_step(opt, micro_batch, acc, 0.05, loss_grad=loss_grad, fused_clip=fused,
+                                        freeze=[st.grad(emb)])
+    torch.cuda.synchronize()
+    assert loss == 2.0
+    hs[emb]["g"][...] = 0
+    sq = sum(float((O.h2f(h["g"]).astype(np.float64) ** 2).sum()) if h["g"].dtype == np.uint16
+             else float((h["g"].astype(np.float64) ** 2).sum()) for h in hs)
+    assert abs(norm - math.sqrt(sq)) <= 1e-5 * math.sqrt(sq) and norm > 0.05
+    _, s_dev, _ = opt.plan.norm_read()
+    assert not st.grad(emb).any().item()
+    if not fused:                                     # the scale pass rewrote the gradients: compare them too
+        for i, h in enumerate(hs):
+            exp = h["g"].copy()
+            (O.scale_half if exp.dtype == np.uint16 else O.scale_float)(exp, s_dev)
+            assert np.array_equal(bits(st.grad(i)), exp), "scaled gradients, tensor %d" % i
+    oracle_step(O, L, specs, hs, 1, dict(HYPER, lr=1e-3), clip_scale=s_dev)
+    assert compare(st, hs, "accumulation step") == 0
