@@ -203,7 +203,8 @@ int rlx_plan_adamw_dev(rlx_plan* plan, const rlx_step_params* dev_params, int st
 /* ------------------------------------------------------------------------------------
  * Launch tuning (process-wide; for measurement).  Unknown keys return RLX_ERR_INVALID_ARG.
  *   "update_variant"  0..N-1   which compiled form of the update kernel: tile shape, XCD swizzle,
- *                              store policy (0 = default)
+ *                              store policy, loads and stores at once or two at a time (0 = default,
+ *                              which picks between the last two by what the step writes)
  *   "norm_grid"       0 = one workgroup per chunk, >0 = that many persistent workgroups
  *   "norm_nt"         1 = non-temporal loads in the norm pass (default), 0 = plain
  * ---------------------------------------------------------------------------------- */

@@ -286,23 +286,32 @@ def test_ragged_list_equals_flat_tensor(O, L, host, B, torch_gpu):
     assert not st.m[~used].any().item() and not st.p16[~used[: st.p16.numel()]].any().item()
 
 
-def test_every_tile_shape_and_chunk_size_gives_the_same_bits(L, host, B, torch_gpu):
+@pytest.mark.parametrize("master,zero_grads", [(False, False), (True, False), (False, True), (True, True)])
+def test_every_tile_shape_and_chunk_size_gives_the_same_bits(L, host, B, torch_gpu, master, zero_grads):
+    """Every compiled form of the update kernel (tile shapes, XCD swizzle, store policy, and the two forms that
+    issue their loads and stores at once or two at a time) gives the same bits, with and without a master copy
+    and gradient clearing (which select between those two forms by default)."""
     torch = torch_gpu
     specs = [L.TensorSpec("a", 70_001, L.DTYPE_F16, 0, 0), L.TensorSpec("b", 2049, L.DTYPE_F32, 0, 0),
              L.TensorSpec("c", 131, L.DTYPE_F16, L.NO_DECAY, 0)]
     results = []
     try:
         for variant, chunk in [(0, 8192), (1, 8192), (2, 2048), (3, 512), (4, 512), (5, 65536), (6, 1024),
-                               (7, 2048)]:
+                               (7, 2048), (8, 8192), (9, 4096)]:
             B.set_tuning("update_variant", variant)
-            st = host.ParamStore(specs)
+            st = host.ParamStore(specs, master=master)
             st.fill("p", 1, 0.0, 0.02)
             st.fill("g", 2, 0.0, 5e-3)
+            if master:
+                st.init_master()
             opt = host.AdamWOptimizer(st, lr=1e-3, chunk_elems=chunk)
-            host.training_step(opt, 0.05, fused_clip=True)
+            host.training_step(opt, 0.05, fused_clip=True, zero_grads=zero_grads)
+            if zero_grads:
+                assert not st.g16.any().item() and not st.g32.any().item()
+                st.fill("g", 3, 0.0, 5e-3)
             host.training_step(opt, 0.0)
             torch.cuda.synchronize()
-            results.append([t.clone() for t in (st.p16, st.p32, st.m, st.v)])
+            results.append([t.clone() for t in (st.p16, st.p32, st.m, st.v)] + ([st.master.clone()] if master else []))
     finally:
         B.set_tuning("update_variant", 0)
     for r in results[1:]:
