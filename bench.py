@@ -326,7 +326,7 @@ def main():
         "hbm_frac_of_peak": BYTES_UPDATE * N * args.steps / wall / 1e9 / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
-                     "kernel": "adamw_tile_kernel<2,128,1,false,1>", "kernel_ms": kernel_ms,
+                     "kernel": "adamw_tile_kernel<2,128,1,false,1,0>", "kernel_ms": kernel_ms,
                      "algorithmic_bytes_per_launch": BYTES_UPDATE * N,
                      "isolated_launch_ms_min": float(np.min(per)), "isolated_launch_ms_median": float(np.median(per))},
         "cpu_baseline": cpu,
