@@ -33,6 +33,7 @@
 #include <cstdio>
 #include <cstring>
 #include <new>
+#include <utility>
 #include <vector>
 
 #include "rlx_adamw.h"
@@ -778,6 +779,23 @@ int flat_update(void* p, const void* g, float* m, float* v, float* master, int64
                                0, master != nullptr, (hipStream_t)stream);
 }
 
+// Zero fill of [dst, dst + nbytes): 128-bit stores over the 16-byte-aligned body, bytes at the edges.
+void clear_range(void* dst, int64_t nbytes, hipStream_t s) {
+    uint8_t* b = (uint8_t*)dst;
+    int64_t n_head = (int64_t)((16 - ((uintptr_t)b & 15)) & 15);
+    if (n_head > nbytes) n_head = nbytes;
+    const int64_t n_vec = (nbytes - n_head) / 16;
+    const int64_t n_tail = nbytes - n_head - n_vec * 16;
+    u32x4* body = (u32x4*)(b + n_head);
+    const int64_t per_launch = kMaxTilesPerLaunch * 256;         // vectors per launch
+    for (int64_t first = 0; first < n_vec; first += per_launch) {
+        const int64_t here = n_vec - first < per_launch ? n_vec - first : per_launch;
+        clear_body_kernel<<<dim3((unsigned)((here + 255) / 256)), dim3(256), 0, s>>>(body + first, here);
+    }
+    if (n_head || n_tail)
+        clear_edges_kernel<<<dim3(1), dim3(64), 0, s>>>(b, (int)n_head, b + n_head + n_vec * 16, (int)n_tail);
+}
+
 }  // namespace
 
 struct rlx_plan {
@@ -786,7 +804,13 @@ struct rlx_plan {
     int chunk_log2;
     bool any_master;         // some tensor has an FP32 master copy
     int64_t n_tensors, n_chunks, n_elems, chunk_elems;
-    ChunkRec* d_recs;
+    ChunkRec* d_recs;        // every chunk, in tensor order (the order of the norm)
+    ChunkRec* d_active;      // the chunks that the update changes (not frozen, not grad-only); == d_recs if all are
+    int64_t n_active;
+    // gradient buffers of the frozen and grad-only tensors, for steps that clear gradients; empty if there are
+    // more than kMaxIdleRanges of them (such steps then run over the full table)
+    std::vector<std::pair<void*, int64_t>> idle_grads;
+    bool idle_by_range;
     double* d_partials;
     NormResult* d_norm;
     NormResult* h_norm;      // pinned
@@ -794,6 +818,7 @@ struct rlx_plan {
 
 namespace {
 constexpr uint32_t kPlanMagic = 0x524C5850u;   // "RLXP"
+constexpr size_t kMaxIdleRanges = 16;
 inline bool plan_ok(const rlx_plan* p) { return p && p->magic == kPlanMagic; }
 
 // A plan's tables and every pointer in them belong to the device that was current when the plan
@@ -816,6 +841,29 @@ void launch_scale_groups(const rlx_plan* p, hipStream_t s) {
         scale_group_kernel<BLOCK><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(p->d_recs, first, n_tiles, tpc_log2,
                                                                              p->d_norm);
     }
+}
+
+// The update launch of a plan.  Frozen and grad-only chunks have nothing to update, and a workgroup that only
+// learns that from its record still costs its dispatch (0.3 ms for the frozen embedding of Qwen3-0.6B), so the
+// update runs over the table without them; a step that clears gradients clears theirs by range.
+int plan_update(const rlx_plan* p, const Hyper& h, const rlx_step_params* dev_params, int step_flags, hipStream_t s) {
+    ChunkRec none;
+    memset(&none, 0, sizeof(none));
+    const NormResult* norm = (step_flags & RLX_CLIP_FUSED) ? p->d_norm : nullptr;
+    const bool clear = (step_flags & RLX_STEP_ZERO_GRADS) != 0;
+    if (clear && !p->idle_by_range)
+        return launch_update<false>(p->d_recs, none, 0, p->n_chunks, p->chunk_log2, h, dev_params, norm,
+                                    (uint32_t)step_flags, p->any_master, s);
+    if (p->n_active > 0) {
+        const int st = launch_update<false>(p->d_active, none, 0, p->n_active, p->chunk_log2, h, dev_params, norm,
+                                            (uint32_t)step_flags, p->any_master, s);
+        if (st != RLX_OK) return st;
+    }
+    if (clear) {
+        for (const auto& r : p->idle_grads) clear_range(r.first, r.second, s);
+        RLX_HIP(hipGetLastError());
+    }
+    return RLX_OK;
 }
 
 }  // namespace
@@ -884,20 +932,7 @@ int rlx_scale_f32(float* x, float scale, int64_t n, void* stream) {
 int rlx_clear(void* dst, int64_t nbytes, void* stream) {
     if (nbytes <= 0) return RLX_OK;
     if (!dst) return RLX_ERR_INVALID_ARG;
-    hipStream_t s = (hipStream_t)stream;
-    uint8_t* b = (uint8_t*)dst;
-    int64_t n_head = (int64_t)((16 - ((uintptr_t)b & 15)) & 15);
-    if (n_head > nbytes) n_head = nbytes;
-    const int64_t n_vec = (nbytes - n_head) / 16;
-    const int64_t n_tail = nbytes - n_head - n_vec * 16;
-    u32x4* body = (u32x4*)(b + n_head);
-    const int64_t per_launch = kMaxTilesPerLaunch * 256;         // vectors per launch
-    for (int64_t first = 0; first < n_vec; first += per_launch) {
-        const int64_t here = n_vec - first < per_launch ? n_vec - first : per_launch;
-        clear_body_kernel<<<dim3((unsigned)((here + 255) / 256)), dim3(256), 0, s>>>(body + first, here);
-    }
-    if (n_head || n_tail)
-        clear_edges_kernel<<<dim3(1), dim3(64), 0, s>>>(b, (int)n_head, b + n_head + n_vec * 16, (int)n_tail);
+    clear_range(dst, nbytes, (hipStream_t)stream);
     RLX_HIP(hipGetLastError());
     return RLX_OK;
 }
@@ -954,8 +989,17 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
     p->chunk_log2 = __builtin_ctzll((unsigned long long)chunk_elems);
     p->n_tensors = count; p->n_chunks = n_chunks; p->n_elems = n_elems; p->chunk_elems = chunk_elems;
     p->any_master = false;
-    for (int64_t i = 0; i < count; i++) p->any_master = p->any_master || descs[i].master != nullptr;
-    p->d_recs = nullptr; p->d_partials = nullptr; p->d_norm = nullptr; p->h_norm = nullptr;
+    p->idle_by_range = true;
+    for (int64_t i = 0; i < count; i++) {
+        p->any_master = p->any_master || descs[i].master != nullptr;
+        if (descs[i].flags & (RLX_TENSOR_GRAD_ONLY | RLX_TENSOR_FROZEN)) {
+            if (p->idle_grads.size() < kMaxIdleRanges)
+                p->idle_grads.emplace_back(descs[i].grad, descs[i].n * (descs[i].dtype == RLX_DTYPE_F16 ? 2 : 4));
+            else
+                p->idle_by_range = false;
+        }
+    }
+    p->d_recs = nullptr; p->d_active = nullptr; p->n_active = 0; p->d_partials = nullptr; p->d_norm = nullptr; p->h_norm = nullptr;
 
     hipError_t e = hipGetDevice(&p->device);
     if (e == hipSuccess) e = hipMalloc((void**)&p->d_recs, sizeof(ChunkRec) * (size_t)n_chunks);
@@ -963,6 +1007,21 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
     if (e == hipSuccess) e = hipMalloc((void**)&p->d_norm, sizeof(NormResult));
     if (e == hipSuccess) e = hipHostMalloc((void**)&p->h_norm, sizeof(NormResult), hipHostMallocDefault);
     if (e == hipSuccess) e = hipMemcpy(p->d_recs, recs.data(), sizeof(ChunkRec) * (size_t)n_chunks, hipMemcpyHostToDevice);
+    if (e == hipSuccess) {
+        // A workgroup that only finds out from its record that it has nothing to do still costs its dispatch
+        // (0.3 ms for the frozen embedding of Qwen3-0.6B): updates that do not clear gradients run over a
+        // table without such chunks.
+        size_t keep = 0;
+        for (size_t i = 0; i < recs.size(); i++)
+            if (!(recs[i].flags & (RLX_TENSOR_GRAD_ONLY | RLX_TENSOR_FROZEN))) recs[keep++] = recs[i];
+        p->n_active = (int64_t)keep;
+        if (keep == recs.size()) {
+            p->d_active = p->d_recs;
+        } else if (keep > 0) {
+            e = hipMalloc((void**)&p->d_active, sizeof(ChunkRec) * keep);
+            if (e == hipSuccess) e = hipMemcpy(p->d_active, recs.data(), sizeof(ChunkRec) * keep, hipMemcpyHostToDevice);
+        }
+    }
     if (e == hipSuccess) {
         const NormResult init = {0.0, 0.0f, 1.0f};
         *p->h_norm = init;
@@ -982,6 +1041,7 @@ int rlx_plan_destroy(rlx_plan* p) {
     if (!p) return RLX_OK;
     if (!plan_ok(p)) return RLX_ERR_INVALID_ARG;
     hipError_t first = hipSuccess, e;
+    if (p->d_active && p->d_active != p->d_recs && (e = hipFree(p->d_active)) != hipSuccess && first == hipSuccess) first = e;
     if (p->d_recs && (e = hipFree(p->d_recs)) != hipSuccess && first == hipSuccess) first = e;
     if (p->d_partials && (e = hipFree(p->d_partials)) != hipSuccess && first == hipSuccess) first = e;
     if (p->d_norm && (e = hipFree(p->d_norm)) != hipSuccess && first == hipSuccess) first = e;
@@ -1054,11 +1114,7 @@ int rlx_plan_adamw(rlx_plan* p, const rlx_step_params* sp, int step_flags, void*
     if (st != RLX_OK) return st;
     const Hyper h = make_hyper(sp->lr, sp->beta1, sp->beta2, sp->eps, sp->weight_decay, sp->bias_correction1,
                                sp->bias_correction2);
-    ChunkRec none;
-    memset(&none, 0, sizeof(none));
-    return launch_update<false>(p->d_recs, none, 0, p->n_chunks, p->chunk_log2, h, nullptr,
-                                (step_flags & RLX_CLIP_FUSED) ? p->d_norm : nullptr, (uint32_t)step_flags,
-                                p->any_master, (hipStream_t)stream);
+    return plan_update(p, h, nullptr, step_flags, (hipStream_t)stream);
 }
 
 int rlx_plan_adamw_dev(rlx_plan* p, const rlx_step_params* dev_params, int step_flags, void* stream) {
@@ -1067,13 +1123,9 @@ int rlx_plan_adamw_dev(rlx_plan* p, const rlx_step_params* dev_params, int step_
     if (!is_aligned(dev_params, 4)) return RLX_ERR_MISALIGNED;
     const int ready = plan_launchable(p);
     if (ready != RLX_OK) return ready;
-    ChunkRec none;
-    memset(&none, 0, sizeof(none));
     Hyper h;
     memset(&h, 0, sizeof(h));
-    return launch_update<false>(p->d_recs, none, 0, p->n_chunks, p->chunk_log2, h, dev_params,
-                                (step_flags & RLX_CLIP_FUSED) ? p->d_norm : nullptr, (uint32_t)step_flags,
-                                p->any_master, (hipStream_t)stream);
+    return plan_update(p, h, dev_params, step_flags, (hipStream_t)stream);
 }
 
 int rlx_set_tuning(const char* key, int64_t value) {
