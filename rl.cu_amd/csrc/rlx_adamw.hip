@@ -232,6 +232,9 @@ __device__ __forceinline__ void update_scalar32(const ChunkRec& r, int64_t i, co
 // K > 1: workgroups b, b+8, ... land on the same XCD; groups of 8*K tiles are permuted so
 // that each XCD gets K neighbouring tiles.
 // SINGLE: one flat tensor passed by value (the operator API); otherwise the plan's records.
+// SP: 1 = system-scope non-temporal stores, 0 = plain non-temporal stores.
+// PH: 0 = a lane issues the tile's four loads at once; 1 = tiles that write four streams (master copy,
+// gradient clearing) issue their loads, and with a master copy their stores, two at a time.
 // ---------------------------------------------------------------------------------------
 
 template <int E, int BLOCK, int K, bool SINGLE, int SP, int PH>
