@@ -536,12 +536,13 @@ def test_element_by_element_paths_with_master_fp32_and_half_precision_workspace(
 
 @pytest.mark.parametrize("seed", list(range(int(os.environ.get("RLX_RANDOM_PLAN_SEEDS", "12")))))
 def test_random_plans(O, L, host, B, torch_gpu, seed):
-    """Seeded random tensor lists: sizes from 1 to 70,000, both dtypes, any start alignment, master copy or
+    """Seeded random tensor lists (1 to 13 tensors, one list in four 30 to 69 so that more than 16 of them are
+    frozen or grad-only, the limit up to which their gradients are cleared by range): sizes from 1 to 70,000, both dtypes, any start alignment, master copy or
     not, no-decay / frozen / grad-only flags, every chunk size, two steps with norm, fused or unfused clip
     and optional gradient clearing; every byte of every buffer (guard zones included) against the oracle."""
     torch = torch_gpu
     rng = np.random.default_rng(1000 + seed)
-    count = int(rng.integers(1, 14))
+    count = int(rng.integers(1, 14)) if rng.integers(0, 4) else int(rng.integers(30, 70))   # many: more than 16
     chunk = int(rng.choice([512, 1024, 2048, 4096, 8192, 32768]))
     fused = bool(rng.integers(0, 2))
     zero = bool(rng.integers(0, 2))
