@@ -158,6 +158,12 @@ def clip_grad_norm(half_pool, float_pool, max_norm):
     return float(norm), float(sc.value)
 
 
+def sumsq_mirror_final(partials):
+    """The fixed-order FP64 sum of per-chunk partials (pass 2 of the device's norm)."""
+    allp = np.ascontiguousarray(partials, dtype=np.float64)
+    return float(lib.orc_sumsq_mirror_final(_p(allp, F64), allp.size))
+
+
 def sumsq_mirror(grads, chunk):
     """Sum of squares of a list of gradient arrays in the device's reduction order."""
     parts = []

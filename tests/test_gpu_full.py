@@ -5,7 +5,7 @@ checked on the device."""
 import numpy as np
 import pytest
 
-from util import bits
+from util import bits, read_device
 
 pytestmark = pytest.mark.gpu
 
@@ -168,6 +168,27 @@ def test_qwen3_8b_resident(O, L, host, torch_gpu):
     # a second, identical run of the norm gives the same bits
     opt.plan.grad_norm(1.0)
     assert opt.plan.norm_read() == (n2, scale, sum_sq)
+    # the million per-chunk partials: their fixed-order sum is the result, and sampled chunks (random ones, the
+    # last and possibly short chunk of every tensor, chunks whose elements lie beyond index 2^32) equal the
+    # restated reduction order on gradients regenerated on the host
+    chunk = opt.plan.chunk_elems
+    parts = read_device(opt.plan.partials_ptr, 8 * opt.plan.num_chunks).view(np.float64)
+    assert O.sumsq_mirror_final(parts) == sum_sq
+    first_chunk = np.cumsum([0] + [-(-s.n // chunk) for s in specs])
+    assert first_chunk[-1] == opt.plan.num_chunks
+    rng = np.random.default_rng(11)
+    picks = [(i, int(first_chunk[i + 1] - first_chunk[i]) - 1) for i in range(len(specs))]
+    picks += [(int(i), int(rng.integers(0, first_chunk[i + 1] - first_chunk[i]))) for i in rng.integers(0, len(specs), 200)]
+    beyond = 0
+    for i, c in picks:
+        lo = c * chunk
+        n = min(chunk, specs[i].n - lo)
+        beyond += st.off[i] + lo > 2 ** 32
+        g = O.fill_f16(n, L._hash64(0x5EED0011, i), 0.0, 1e-4, first=lo)
+        _, one = O.sumsq_mirror([g], chunk)
+        got = parts[first_chunk[i] + c]
+        assert one.size == 1 and one.view(np.uint64)[0] == np.float64(got).view(np.uint64), "tensor %d chunk %d" % (i, c)
+    assert beyond > 100
 
 
 def test_single_tensor_beyond_int32(O, B, host, torch_gpu):
