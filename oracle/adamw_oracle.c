@@ -14,7 +14,8 @@
  *   orc_fp16_to_fp32      include/training/optimizer.h:46-57
  *   orc_sum_sq_half/float include/training/trainer.h:103-133 (sum of squares; accumulated here in FP64,
  *                         the reference accumulates in FP32 with unordered atomics)
- *   orc_scale_half/float  include/training/trainer.h:136-145
+ *   orc_scale_half/float  include/training/trainer.h:136-145 (orc_scale_float is also the arithmetic of
+ *                         scale_grad_kernel, trainer.h:96-99: one FP32 multiply per element)
  *   orc_clip_grad_norm    include/training/trainer.h:323-352
  *
  * Parity pins (tests/test_oracle_*.py): orc_h2f is checked on all 65,536 inputs and
