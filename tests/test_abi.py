@@ -61,6 +61,12 @@ def test_argument_checks_need_no_device(B):
     assert B.adamw_fp32(0x1000, 0x1000, 0x1000, 0x1000, 8, float("inf"), 0.9, 0.999, 1e-8, 0.0, 0.1, 0.1) \
         == B.ERR_BAD_HYPER
     assert B.fp16_to_fp32(0x1000, None, 4) == B.ERR_INVALID_ARG
+    lib = B.load()
+    assert lib.rlx_clear(None, 0, None) == B.OK and lib.rlx_clear(None, -5, None) == B.OK
+    assert lib.rlx_clear(None, 16, None) == B.ERR_INVALID_ARG
+    assert lib.rlx_scale_f32(None, 0.5, 0, None) == B.OK
+    assert lib.rlx_scale_f32(None, 0.5, 4, None) == B.ERR_INVALID_ARG
+    assert lib.rlx_scale_f32(0x1002, 0.5, 4, None) == B.ERR_MISALIGNED
 
 
 def test_plan_argument_checks(B):
