@@ -480,15 +480,19 @@ __global__ __launch_bounds__(kFinalBlock) void sumsq_final_kernel(
     const int tid = threadIdx.x;
     double a = 0.0;
     int64_t i = tid;
-    // sixteen independent loads in flight, added in index order: the same sum as one at a time
-    for (; i + 15 * (int64_t)kFinalBlock < n_partials; i += 16 * (int64_t)kFinalBlock) {
+    // sixteen independent loads in flight, added in index order: the same sum as one at a time.  Slots beyond
+    // the end read as +0.0, which leaves a sum of squares (never negative zero) unchanged bit for bit; without
+    // them the last few partials of every lane would each cost a round trip of their own.
+    for (; i < n_partials; i += 16 * (int64_t)kFinalBlock) {
         double x[16];
 #pragma unroll
-        for (int k = 0; k < 16; k++) x[k] = partials[i + k * (int64_t)kFinalBlock];
+        for (int k = 0; k < 16; k++) {
+            const int64_t j = i + k * (int64_t)kFinalBlock;
+            x[k] = j < n_partials ? partials[j] : 0.0;
+        }
 #pragma unroll
         for (int k = 0; k < 16; k++) a += x[k];
     }
-    for (; i < n_partials; i += kFinalBlock) a += partials[i];
     acc[tid] = a;
     __syncthreads();
     for (int s = kFinalBlock / 2; s >= 1; s >>= 1) {
