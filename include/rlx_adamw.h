@@ -123,8 +123,9 @@ typedef struct rlx_plan rlx_plan;
  * Builds the device-resident work table for `count` tensors (the role that
  * AdamWOptimizer::init's offset bookkeeping has, include/training/optimizer.h:188-243).
  * Tensors are cut into chunks of `chunk_elems` elements (0 = chosen from the mean tensor
- * size: 8192, 2048 or 512; otherwise a power of two >= 512); the table order is the order of
- * `descs`, which also fixes the order of the norm reduction.  The plan borrows every pointer in `descs` and owns only
+ * size: 8192, 2048 or 512, and up to 65536 for lists of billions of elements; otherwise a
+ * power of two >= 512); the table order is the order of `descs`, which also fixes the order
+ * of the norm reduction.  The plan borrows every pointer in `descs` and owns only
  * its tables and the reduction workspace.  Allocates; call outside the step loop.
  */
 int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_elems, rlx_plan** out);

@@ -958,6 +958,9 @@ int rlx_plan_layout(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
     if (chunk_elems == 0) {
         const int64_t mean = n_elems / count;
         chunk_elems = mean >= 4 * kBigChunk ? kBigChunk : mean >= 4 * kSmallChunk ? kSmallChunk : kMinChunk;
+        // very large lists: keep the number of partials that the single-workgroup second pass of the norm
+        // has to read near 2^18 (the update is equally fast with chunks from 8,192 to 65,536 elements)
+        while (chunk_elems >= kBigChunk && chunk_elems < 65536 && n_elems / chunk_elems > (1 << 18)) chunk_elems *= 2;
     }
     if (chunk_elems < kMinChunk || chunk_elems > (1 << 24) || (chunk_elems & (chunk_elems - 1)) != 0)
         return RLX_ERR_INVALID_ARG;
