@@ -26,7 +26,7 @@ typedef enum {
     RLX_ERR_BAD_HYPER = 3,        /* bias correction of 0, or a non-finite hyper-parameter */
     RLX_ERR_HIP = 4,              /* a HIP runtime call failed; see rlx_last_hip_error() */
     RLX_ERR_NO_DEVICE = 5,
-    RLX_ERR_TOO_LARGE = 6,        /* more chunks than one plan can address */
+    RLX_ERR_TOO_LARGE = 6,        /* more chunks than one plan can address, or than rlx_grad_norm_static holds */
     RLX_ERR_NO_MEMORY = 7,        /* host allocation failed */
     RLX_ERR_WRONG_DEVICE = 8      /* the plan was made with another device current */
 } rlx_status;
@@ -167,6 +167,24 @@ int rlx_plan_norm_read(rlx_plan* plan, float* norm, float* scale, double* sum_sq
 const void* rlx_plan_norm_device_ptr(const rlx_plan* plan);
 /* Device address of the per-chunk FP64 partials (rlx_plan_num_chunks values). */
 const double* rlx_plan_partials_device_ptr(const rlx_plan* plan);
+
+/*
+ * The same two-pass norm and clip rule over two flat gradient buffers (an FP16 one, then an FP32 one: the
+ * shape of half_pool / float_pool) without a plan and without allocating anything.  It has no counterpart
+ * in the reference; it is for callers that cannot allocate: code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc.  The per-chunk FP64 partials go to a 2 MiB array that is part of
+ * the library's device image (every GPU the library runs on holds it until the process ends), so at most
+ * 262,144 chunks fit: more returns RLX_ERR_TOO_LARGE (chunk_elems = 0 chooses the chunk as rlx_plan_create
+ * would for these two tensors, which covers about 17e9 elements; otherwise a power of two >= 512).
+ * Writes {double sum_sq; float norm; float scale;} (16 bytes, 8-byte aligned, device) to result_dev: the same
+ * bits as rlx_plan_grad_norm leaves for a plan over these two tensors in this order with the same chunk size.
+ * Either buffer may be empty (n = 0).  Calls no hipMalloc, hipFree or other allocating routine; the first call
+ * on a device looks up the array's address there (make that call outside a graph capture).  All calls on one
+ * GPU share the array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream
+ * do not.  Nothing in the array has to start at zero: every call writes each slot that it later reads.
+ */
+int rlx_grad_norm_static(const uint16_t* half_grads, int64_t n_half, const float* float_grads, int64_t n_float,
+                         int64_t chunk_elems, float max_norm, void* result_dev, void* stream);
 
 /*
  * In-place scale of all gradients by the device-resident clip scale: replaces

@@ -54,6 +54,7 @@ SIGNATURES = {
     "rlx_plan_num_elements": ([_VP], _I64),
     "rlx_plan_chunk_elems": ([_VP], _I64),
     "rlx_plan_grad_norm": ([_VP, _F, _VP], _INT),
+    "rlx_grad_norm_static": ([_VP, _I64, _VP, _I64, _I64, _F, _VP, _VP], _INT),
     "rlx_plan_norm_read": ([_VP, C.POINTER(_F), C.POINTER(_F), C.POINTER(C.c_double), _VP], _INT),
     "rlx_plan_norm_device_ptr": ([_VP], _VP),
     "rlx_plan_partials_device_ptr": ([_VP], _VP),
@@ -151,6 +152,13 @@ def clear(dst, nbytes, stream=0):
 
 def scale_f32(x, scale, n, stream=0):
     check(load().rlx_scale_f32(x, scale, n, stream), "rlx_scale_f32")
+
+
+def grad_norm_static(half_grads, n_half, float_grads, n_float, max_norm, result_dev, chunk_elems=0, stream=0):
+    """Norm and clip scale of two flat gradient buffers into 16 bytes at result_dev; allocates nothing.
+    Returns the status."""
+    return load().rlx_grad_norm_static(half_grads, n_half, float_grads, n_float, chunk_elems, max_norm, result_dev,
+                                       stream)
 
 
 def plan_layout(descs, chunk_elems=0):

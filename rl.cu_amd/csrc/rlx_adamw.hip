@@ -32,11 +32,19 @@
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 #include <utility>
 #include <vector>
 
 #include "rlx_adamw.h"
+
+// Per-chunk FP64 partials of rlx_grad_norm_static, the entry point for callers that cannot allocate: part of
+// the library's device image (2 MiB on every GPU the library runs on, until the process ends).  The name
+// stands for the array only in device code; host code uses the address that hipGetSymbolAddress returns for
+// the current device (static_scratch below), never the name.
+constexpr int64_t kStaticMaxPartials = 1 << 18;
+static __device__ __align__(256) double scratch[kStaticMaxPartials];
 
 namespace {
 
@@ -77,6 +85,18 @@ struct NormResult {
 
 struct Hyper {
     float lr, beta1, beta2, eps, weight_decay, bc1_inv, bc2_inv;
+};
+
+// Two flat gradient buffers described by value (an FP16 one followed by an FP32 one, the shape of
+// the reference's half_pool / float_pool): the chunks that a plan over these two tensors would
+// hold, without a table in device memory.
+struct PoolPair {
+    const uint16_t* half_pool;
+    const float* float_pool;
+    int64_t n_half, n_float;
+    int64_t chunks_half;             // chunks of the FP16 buffer; those of the FP32 buffer follow
+    int chunk_log2;
+    uint32_t flags_half, flags_float;   // ChunkRec::flags of every chunk of the buffer
 };
 
 // ---------------------------------------------------------------------------------------
@@ -384,16 +404,37 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
 // two 128-bit reads each measured 7.3 TB/s as a stand-alone stream, 256 lanes with four 6.95.)
 // ---------------------------------------------------------------------------------------
 
-template <bool NT, int BLOCK>
+// Chunk c of a PoolPair as the record that a plan would hold for it (only the fields the norm reads).
+__device__ __forceinline__ ChunkRec pool_chunk(const PoolPair& pp, int64_t c) {
+    ChunkRec r;
+    const int64_t chunk = (int64_t)1 << pp.chunk_log2;
+    if (c < pp.chunks_half) {
+        const int64_t start = c << pp.chunk_log2, left = pp.n_half - start;
+        r.g = (void*)(pp.half_pool + start);
+        r.count = (uint32_t)(left < chunk ? left : chunk);
+        r.flags = pp.flags_half;
+    } else {
+        const int64_t start = (c - pp.chunks_half) << pp.chunk_log2, left = pp.n_float - start;
+        r.g = (void*)(pp.float_pool + start);
+        r.count = (uint32_t)(left < chunk ? left : chunk);
+        r.flags = pp.flags_float;
+    }
+    return r;
+}
+
+// POOLS: the chunks come from `pools` (two flat buffers passed by value) instead of the table `recs`.
+template <bool NT, int BLOCK, bool POOLS = false>
 __global__ __launch_bounds__(BLOCK) void sumsq_partials_kernel(
-    const ChunkRec* __restrict__ recs, int64_t n_chunks, double* __restrict__ partials)
+    const ChunkRec* __restrict__ recs, PoolPair pools, int64_t n_chunks, double* __restrict__ partials)
 {
     constexpr int kNormGroup = BLOCK * kVec;
     __shared__ float wave_sum[BLOCK / 64];
     const int tid = threadIdx.x;
 
     for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
-        const ChunkRec r = recs[c];
+        ChunkRec r;
+        if constexpr (POOLS) r = pool_chunk(pools, c);
+        else r = recs[c];
         const int64_t count = r.count;
         const bool aligned = ((r.flags >> kValignShift) & 0xF) >= 8;
 
@@ -645,6 +686,10 @@ __global__ __launch_bounds__(kFillBlock) void fill_kernel(T* __restrict__ dst, i
 
 thread_local char g_hip_error[256] = "";
 
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+double* g_scratch_ptr[kMaxDevices];      // device address of `scratch` on each device; null until first used there
+
 int hip_fail(hipError_t e, const char* what) {
     snprintf(g_hip_error, sizeof(g_hip_error), "%s: %s", what, hipGetErrorString(e));
     return RLX_ERR_HIP;
@@ -697,6 +742,19 @@ int check_desc(const rlx_tensor_desc& d) {
         return RLX_ERR_MISALIGNED;
     return RLX_OK;
 }
+
+// Default chunk size: big chunks for big tensors; for a list of many small tensors a smaller chunk
+// wastes fewer workgroups on the empty part of each tensor's last chunk.
+int64_t default_chunk(int64_t n_elems, int64_t n_tensors) {
+    const int64_t mean = n_elems / n_tensors;
+    int64_t chunk = mean >= 4 * kBigChunk ? kBigChunk : mean >= 4 * kSmallChunk ? kSmallChunk : kMinChunk;
+    // very large lists: keep the number of partials that the single-workgroup second pass of the norm
+    // has to read near 2^18 (the update is equally fast with chunks from 8,192 to 65,536 elements)
+    while (chunk >= kBigChunk && chunk < 65536 && n_elems / chunk > (1 << 18)) chunk *= 2;
+    return chunk;
+}
+
+inline bool chunk_ok(int64_t chunk) { return chunk >= kMinChunk && chunk <= (1 << 24) && (chunk & (chunk - 1)) == 0; }
 
 // Record of the chunk that starts `start` elements into the tensor.
 ChunkRec make_rec(const rlx_tensor_desc& d, int64_t start, int64_t count) {
@@ -850,6 +908,34 @@ void launch_scale_groups(const rlx_plan* p, hipStream_t s) {
     }
 }
 
+// Both passes of the norm over n_chunks chunks (from the table `recs`, or from `pools` if POOLS): one FP64
+// partial per chunk into `partials`, then the fixed-order sum and the clip rule into `result`.
+template <bool POOLS>
+int launch_norm(const ChunkRec* recs, const PoolPair& pools, int64_t n_chunks, int64_t chunk_elems, double* partials,
+                float max_norm, NormResult* result, hipStream_t s) {
+    int64_t g = g_tuning.norm_grid > 0 ? g_tuning.norm_grid : n_chunks;
+    if (g > n_chunks) g = n_chunks;
+    if (g > kMaxNormGrid) g = kMaxNormGrid;
+    const dim3 grid((unsigned)g);
+    const int64_t lanes = chunk_elems / kVec < kNormBlock ? chunk_elems / kVec : kNormBlock;
+#define RLX_NORM_LAUNCH(BLOCK)                                                                                       \
+    do {                                                                                                             \
+        if (g_tuning.norm_nt)                                                                                        \
+            sumsq_partials_kernel<true, BLOCK, POOLS><<<grid, dim3(BLOCK), 0, s>>>(recs, pools, n_chunks, partials);  \
+        else                                                                                                         \
+            sumsq_partials_kernel<false, BLOCK, POOLS><<<grid, dim3(BLOCK), 0, s>>>(recs, pools, n_chunks, partials); \
+    } while (0)
+    if (lanes >= 512) RLX_NORM_LAUNCH(512);
+    else if (lanes == 256) RLX_NORM_LAUNCH(256);
+    else if (lanes == 128) RLX_NORM_LAUNCH(128);
+    else RLX_NORM_LAUNCH(64);
+#undef RLX_NORM_LAUNCH
+    RLX_HIP(hipGetLastError());
+    sumsq_final_kernel<<<dim3(1), dim3(kFinalBlock), 0, s>>>(partials, n_chunks, max_norm, result);
+    RLX_HIP(hipGetLastError());
+    return RLX_OK;
+}
+
 // The update launch of a plan.  Frozen and grad-only chunks have nothing to update, and a workgroup that only
 // learns that from its record still costs its dispatch (0.3 ms for the frozen embedding of Qwen3-0.6B), so the
 // update runs over the table without them; a step that clears gradients clears theirs by range.
@@ -885,7 +971,7 @@ const char* rlx_status_string(int status) {
     case RLX_ERR_BAD_HYPER: return "bias correction is zero or a hyper-parameter is not finite";
     case RLX_ERR_HIP: return "HIP runtime error";
     case RLX_ERR_NO_DEVICE: return "no HIP device";
-    case RLX_ERR_TOO_LARGE: return "too many chunks for one plan";
+    case RLX_ERR_TOO_LARGE: return "too many chunks: more than one plan can address, or more than the 262,144 partials that the static scratch of rlx_grad_norm_static holds";
     case RLX_ERR_NO_MEMORY: return "out of host memory";
     case RLX_ERR_WRONG_DEVICE: return "the plan belongs to another device than the current one";
     default: return "unknown status";
@@ -894,7 +980,7 @@ const char* rlx_status_string(int status) {
 
 const char* rlx_last_hip_error(void) { return g_hip_error; }
 
-int rlx_version(void) { return 106; }
+int rlx_version(void) { return 107; }
 
 int rlx_adamw_fp16(float* master_w, uint16_t* model_w, const uint16_t* grad, float* m, float* v, int64_t n,
                    float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -953,17 +1039,8 @@ int rlx_plan_layout(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
         if (st != RLX_OK) return st;
         n_elems += descs[i].n;
     }
-    // Default: big chunks for big tensors; for a list of many small tensors a smaller chunk
-    // wastes fewer workgroups on the empty part of each tensor's last chunk.
-    if (chunk_elems == 0) {
-        const int64_t mean = n_elems / count;
-        chunk_elems = mean >= 4 * kBigChunk ? kBigChunk : mean >= 4 * kSmallChunk ? kSmallChunk : kMinChunk;
-        // very large lists: keep the number of partials that the single-workgroup second pass of the norm
-        // has to read near 2^18 (the update is equally fast with chunks from 8,192 to 65,536 elements)
-        while (chunk_elems >= kBigChunk && chunk_elems < 65536 && n_elems / chunk_elems > (1 << 18)) chunk_elems *= 2;
-    }
-    if (chunk_elems < kMinChunk || chunk_elems > (1 << 24) || (chunk_elems & (chunk_elems - 1)) != 0)
-        return RLX_ERR_INVALID_ARG;
+    if (chunk_elems == 0) chunk_elems = default_chunk(n_elems, count);
+    if (!chunk_ok(chunk_elems)) return RLX_ERR_INVALID_ARG;
     int64_t n_chunks = 0;
     for (int64_t i = 0; i < count; i++) n_chunks += (descs[i].n + chunk_elems - 1) / chunk_elems;
     if (n_chunks > INT32_MAX) return RLX_ERR_TOO_LARGE;
@@ -1070,28 +1147,61 @@ const double* rlx_plan_partials_device_ptr(const rlx_plan* p) { return plan_ok(p
 int rlx_plan_grad_norm(rlx_plan* p, float max_norm, void* stream) {
     const int ready = plan_launchable(p);
     if (ready != RLX_OK) return ready;
-    hipStream_t s = (hipStream_t)stream;
-    int64_t g = g_tuning.norm_grid > 0 ? g_tuning.norm_grid : p->n_chunks;
-    if (g > p->n_chunks) g = p->n_chunks;
-    if (g > kMaxNormGrid) g = kMaxNormGrid;
-    const dim3 grid((unsigned)g);
-    const int64_t lanes = p->chunk_elems / kVec < kNormBlock ? p->chunk_elems / kVec : kNormBlock;
-#define RLX_NORM_LAUNCH(BLOCK)                                                                                   \
-    do {                                                                                                         \
-        if (g_tuning.norm_nt)                                                                                    \
-            sumsq_partials_kernel<true, BLOCK><<<grid, dim3(BLOCK), 0, s>>>(p->d_recs, p->n_chunks, p->d_partials);  \
-        else                                                                                                     \
-            sumsq_partials_kernel<false, BLOCK><<<grid, dim3(BLOCK), 0, s>>>(p->d_recs, p->n_chunks, p->d_partials); \
-    } while (0)
-    if (lanes >= 512) RLX_NORM_LAUNCH(512);
-    else if (lanes == 256) RLX_NORM_LAUNCH(256);
-    else if (lanes == 128) RLX_NORM_LAUNCH(128);
-    else RLX_NORM_LAUNCH(64);
-#undef RLX_NORM_LAUNCH
-    RLX_HIP(hipGetLastError());
-    sumsq_final_kernel<<<dim3(1), dim3(kFinalBlock), 0, s>>>(p->d_partials, p->n_chunks, max_norm, p->d_norm);
-    RLX_HIP(hipGetLastError());
+    PoolPair none;
+    memset(&none, 0, sizeof(none));
+    return launch_norm<false>(p->d_recs, none, p->n_chunks, p->chunk_elems, p->d_partials, max_norm, p->d_norm,
+                              (hipStream_t)stream);
+}
+
+/* Device address of the static scratch array on the current device, resolved once per device. */
+static int static_scratch(double** out) {
+    int dev = -1;
+    RLX_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return RLX_ERR_INVALID_ARG;
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (!g_scratch_ptr[dev]) {
+        void* ptr = nullptr;
+        RLX_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return RLX_ERR_HIP;
+        g_scratch_ptr[dev] = (double*)ptr;
+    }
+    *out = g_scratch_ptr[dev];
     return RLX_OK;
+}
+
+int rlx_grad_norm_static(const uint16_t* half_grads, int64_t n_half, const float* float_grads, int64_t n_float,
+                         int64_t chunk_elems, float max_norm, void* result_dev, void* stream) {
+    if (n_half < 0 || n_float < 0 || !result_dev) return RLX_ERR_INVALID_ARG;
+    if ((n_half > 0 && !half_grads) || (n_float > 0 && !float_grads)) return RLX_ERR_INVALID_ARG;
+    if (!is_aligned(half_grads, 2) || !is_aligned(float_grads, 4) || !is_aligned(result_dev, 8)) return RLX_ERR_MISALIGNED;
+    const int64_t n_tensors = (n_half > 0) + (n_float > 0);
+    if (chunk_elems == 0) chunk_elems = n_tensors ? default_chunk(n_half + n_float, n_tensors) : kBigChunk;
+    if (!chunk_ok(chunk_elems)) return RLX_ERR_INVALID_ARG;
+    PoolPair pp;
+    pp.half_pool = half_grads; pp.float_pool = float_grads; pp.n_half = n_half; pp.n_float = n_float;
+    pp.chunk_log2 = __builtin_ctzll((unsigned long long)chunk_elems);
+    pp.chunks_half = (n_half + chunk_elems - 1) / chunk_elems;
+    const int64_t n_chunks = pp.chunks_half + (n_float + chunk_elems - 1) / chunk_elems;
+    if (n_chunks > kStaticMaxPartials) return RLX_ERR_TOO_LARGE;
+    // the flags that a plan's record of a gradient-only tensor at this address would carry
+    rlx_tensor_desc d;
+    memset(&d, 0, sizeof(d));
+    d.flags = RLX_TENSOR_GRAD_ONLY;
+    d.grad = const_cast<uint16_t*>(half_grads); d.dtype = RLX_DTYPE_F16;
+    pp.flags_half = make_rec(d, 0, 0).flags;
+    d.grad = const_cast<float*>(float_grads); d.dtype = RLX_DTYPE_F32;
+    pp.flags_float = make_rec(d, 0, 0).flags;
+    double* partials = nullptr;
+    const int st = static_scratch(&partials);
+    if (st != RLX_OK) return st;
+    if (n_chunks == 0) {      // nothing to add up: sum 0, norm 0, scale by the rule
+        sumsq_final_kernel<<<dim3(1), dim3(kFinalBlock), 0, (hipStream_t)stream>>>(partials, 0, max_norm,
+                                                                                   (NormResult*)result_dev);
+        RLX_HIP(hipGetLastError());
+        return RLX_OK;
+    }
+    return launch_norm<true>(nullptr, pp, n_chunks, chunk_elems, partials, max_norm, (NormResult*)result_dev,
+                             (hipStream_t)stream);
 }
 
 int rlx_plan_norm_read(rlx_plan* p, float* norm, float* scale, double* sum_sq, void* stream) {
