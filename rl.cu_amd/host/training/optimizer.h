@@ -1,5 +1,10 @@
 // AdamWOptimizer for C++ callers: the reference's class (include/training/optimizer.h:59-274)
-// with the same public members and methods, built from flat pools instead of a Qwen3Model*.
+// with the same public members and methods.  It is built either from flat pools (ParamPools) or, with the
+// reference's own constructor signature, from a pointer to any model type that has the members the
+// reference's constructor reads (model->config.* and model->weights.fp16_pool / fp32_pool / *_elems);
+// step() and clip_grad_norm_() take a pointer to any gradient type with half_pool / float_pool /
+// half_pool_bytes / float_pool_bytes, so the reference's call sites (optimizer_(model, ...),
+// clip_grad_norm_(grads_, max), optimizer_.step(grads_)) compile as they stand.
 //
 // Like the reference it owns the FP32 state as flat buffers co-indexed with the weight pools:
 // [master | m | v] for the FP16 pool and [m | v] for the FP32 pool, zero-filled, master
@@ -13,6 +18,8 @@
 #include <cstdint>
 #include <cstring>
 #include <string>
+#include <type_traits>
+#include <utility>
 #include <vector>
 
 #include "../kernels/adamw.h"
@@ -138,6 +145,29 @@ public:
         init(pools, use_master);
     }
 
+    // The reference's constructor (optimizer.h:70-80) for any model type with the members it reads:
+    // model->config.{num_hidden_layers, hidden_size, q_dim, kv_dim, intermediate_size, head_dim, vocab_size}
+    // and model->weights.{fp16_pool, fp16_pool_elems, fp32_pool, fp32_pool_elems}.  The sizes derived from the
+    // configuration must equal the pool sizes (the reference asserts the same, optimizer.h:221-222).
+    template <class Model, class = decltype(std::declval<Model&>().weights.fp16_pool_elems)>
+    explicit AdamWOptimizer(Model* model, float lr = 1e-4f, float beta1 = 0.9f, float beta2 = 0.999f,
+                            float eps = 1e-8f, float weight_decay = 0.01f, bool use_master = true)
+        : lr(lr), beta1(beta1), beta2(beta2), eps(eps), weight_decay(weight_decay) {
+        const auto& c = model->config;
+        ParamPools pools = ParamPools::for_qwen3(c.num_hidden_layers, c.hidden_size, c.q_dim, c.kv_dim,
+                                                 c.intermediate_size, c.head_dim, c.vocab_size);
+        if (pools.fp16_pool_elems != (size_t)model->weights.fp16_pool_elems ||
+            pools.fp32_pool_elems != (size_t)model->weights.fp32_pool_elems) {
+            fprintf(stderr, "[AdamW] the model's weight pools (%zu FP16, %zu FP32 elements) do not have the sizes that "
+                            "its configuration gives (%zu, %zu)\n", (size_t)model->weights.fp16_pool_elems,
+                    (size_t)model->weights.fp32_pool_elems, pools.fp16_pool_elems, pools.fp32_pool_elems);
+            exit(1);
+        }
+        pools.fp16_pool = model->weights.fp16_pool;
+        pools.fp32_pool = model->weights.fp32_pool;
+        init(pools, use_master);
+    }
+
     ~AdamWOptimizer() { free(); }
 
     AdamWOptimizer(const AdamWOptimizer&) = delete;
@@ -180,10 +210,29 @@ public:
         }
     }
 
-    // One optimizer step.  fused_clip: apply the clip scale that the last norm pass of
-    // plan_for(grads) left on the device, inside the update.  zero_grads: clear both gradient
+    // How the reference's two calls behave here (both off by default, which is the reference's behaviour):
+    // fused clip: clip_grad_norm_() leaves the gradients unscaled and the following step() applies the scale
+    // inside the update (one pass over the gradients less); zero grads: step() clears both gradient pools after
+    // reading them (then the caller drops its qwen3_gradients_zero at the start of the next step).
+    void set_fused_clip(bool on) { fused_clip_ = on; if (!on) clip_pending_ = false; }
+    void set_zero_grads(bool on) { zero_grads_ = on; }
+    bool fused_clip() const { return fused_clip_; }
+
+    // One optimizer step with the reference's signature (optimizer.h:119): step(grads, stream = 0).
+    // `grads` is any type with half_pool, float_pool, half_pool_bytes, float_pool_bytes
+    // (Qwen3Gradients, include/model/qwen3.h:190-218; GradPools above).
+    template <class Grads>
+    void step(Grads* grads, hipStream_t stream = 0) {
+        const bool fused = clip_pending_;
+        clip_pending_ = false;
+        step(grads, stream, fused, zero_grads_);
+    }
+
+    // The same with the two options given per call.  fused_clip: apply the clip scale that the last norm
+    // pass of plan_for(grads) left on the device, inside the update.  zero_grads: clear both gradient
     // pools after they have been read (the job of qwen3_gradients_zero at the next step).
-    void step(GradPools* grads, hipStream_t stream = 0, bool fused_clip = false, bool zero_grads = false) {
+    template <class Grads>
+    void step(Grads* grads, hipStream_t stream, bool fused_clip, bool zero_grads) {
         step_++;
         rlx_step_params sp;
         sp.lr = lr; sp.beta1 = beta1; sp.beta2 = beta2; sp.eps = eps; sp.weight_decay = weight_decay;
@@ -191,6 +240,21 @@ public:
         sp.bias_correction2 = 1.0f - powf(beta2, (float)step_);
         const int flags = (fused_clip ? RLX_CLIP_FUSED : 0) | (zero_grads ? RLX_STEP_ZERO_GRADS : 0);
         RLX_CHECK(rlx_plan_adamw(plan_for(grads), &sp, flags, (void*)stream));
+    }
+
+    // Trainer::clip_grad_norm_ (trainer.h:323-352) over the same gradient type: clips all gradients
+    // (half_pool + float_pool) so that the global L2 norm is <= max_norm and returns the pre-clip norm
+    // (host scalar, synchronous), like the reference.  With set_fused_clip(true) the gradients stay as they
+    // are and the next step() applies the scale.  It lives here because the optimizer owns the plan.
+    template <class Grads>
+    float clip_grad_norm_(Grads* grads, float max_norm, hipStream_t stream = 0) {
+        rlx_plan* plan = plan_for(grads);
+        RLX_CHECK(rlx_plan_grad_norm(plan, max_norm, (void*)stream));
+        float total_norm = 0.0f;
+        RLX_CHECK(rlx_plan_norm_read(plan, &total_norm, nullptr, nullptr, (void*)stream));
+        if (fused_clip_) clip_pending_ = true;
+        else if (total_norm > max_norm) RLX_CHECK(rlx_plan_scale_grads(plan, (void*)stream));
+        return total_norm;
     }
 
     // Optimizer state on disk (the reference's save_checkpoint is a stub, trainer.h:317-319).
@@ -261,7 +325,8 @@ public:
 
     // The multi-tensor plan over {projections, embedding, norm weights, workspace tail} for these
     // gradient pools; built on first use and rebuilt if the pools move.
-    rlx_plan* plan_for(GradPools* grads) {
+    template <class Grads>
+    rlx_plan* plan_for(Grads* grads) {
         if (plan_ && grads->half_pool == plan_half_ && grads->float_pool == plan_float_ &&
             grads->float_pool_bytes == plan_float_bytes_)
             return plan_;
@@ -286,7 +351,7 @@ public:
         }
         const size_t tail = grads->float_pool_bytes / sizeof(float) - n32_;
         if (tail) {
-            d[k++] = {nullptr, grads->float_pool + n32_, nullptr, nullptr, nullptr, (int64_t)tail, RLX_DTYPE_F32,
+            d[k++] = {nullptr, (float*)grads->float_pool + n32_, nullptr, nullptr, nullptr, (int64_t)tail, RLX_DTYPE_F32,
                       RLX_TENSOR_GRAD_ONLY};
         }
         RLX_CHECK(rlx_plan_create(d, k, 0, &plan_));
@@ -310,6 +375,8 @@ private:
     float* plan_float_ = nullptr;
     size_t plan_float_bytes_ = 0;
     bool embed_frozen_ = false;
+    bool fused_clip_ = false, zero_grads_ = false;
+    bool clip_pending_ = false;     // a fused clip_grad_norm_() has run since the last step()
 
     size_t fp16_offset(int layer, int proj) const {
         assert(pools_.num_layers > 0 && layer >= 0 && layer < pools_.num_layers && proj >= 0 && proj < 7);
@@ -360,9 +427,8 @@ private:
                                        (int64_t)n16_, nullptr));
         }
         HIP_CHECK(hipDeviceSynchronize());
-        printf("[AdamW] Flat buffers: fp16=%zu params (%.1f MB state)  fp32=%zu params (%.2f MB state)  "
-               "(lr=%.1e wd=%.2f)\n",
-               n16_, n16_ * parts * sizeof(float) / (1024.0 * 1024.0), n32_,
+        printf("[AdamW] state on device: %zu FP16 params -> %.1f MB (%s), %zu FP32 params -> %.2f MB; lr=%.1e wd=%.2f\n",
+               n16_, n16_ * parts * sizeof(float) / (1024.0 * 1024.0), use_master ? "master, m, v" : "m, v", n32_,
                n32_ * 2 * sizeof(float) / (1024.0 * 1024.0), lr, weight_decay);
     }
 
@@ -382,6 +448,7 @@ private:
         n16_ = o.n16_; n32_ = o.n32_; proj_n_ = o.proj_n_;
         plan_ = o.plan_; plan_half_ = o.plan_half_; plan_float_ = o.plan_float_; plan_float_bytes_ = o.plan_float_bytes_;
         embed_frozen_ = o.embed_frozen_;
+        fused_clip_ = o.fused_clip_; zero_grads_ = o.zero_grads_; clip_pending_ = o.clip_pending_;
         o.plan_ = nullptr; o.fp16_state_ = nullptr; o.fp32_state_ = nullptr;
         o.fp16_master_ = o.fp16_m_ = o.fp16_v_ = o.fp32_m_ = o.fp32_v_ = nullptr;
     }

@@ -25,19 +25,19 @@ public:
 
     // Clip all gradients (half_pool + float_pool) so that the global L2 norm is <= max_norm.
     // Returns the pre-clip norm (host scalar, synchronous), like the reference.
-    float clip_grad_norm_(GradPools* grads, float max_norm, hipStream_t stream = 0) {
-        rlx_plan* plan = optimizer_->plan_for(grads);
-        RLX_CHECK(rlx_plan_grad_norm(plan, max_norm, (void*)stream));
-        float total_norm = 0.0f;
-        RLX_CHECK(rlx_plan_norm_read(plan, &total_norm, nullptr, nullptr, (void*)stream));
-        if (!config_.fused_clip && total_norm > max_norm) RLX_CHECK(rlx_plan_scale_grads(plan, (void*)stream));
-        return total_norm;
+    template <class Grads>
+    float clip_grad_norm_(Grads* grads, float max_norm, hipStream_t stream = 0) {
+        optimizer_->set_fused_clip(config_.fused_clip);
+        return optimizer_->clip_grad_norm_(grads, max_norm, stream);
     }
 
     // What training_step does after the backward passes.  embed_elems: size of the embedding at
     // the end of half_pool (only read when freeze_embed is set).  Returns the pre-clip norm.
-    float apply(GradPools* grads, size_t embed_elems = 0, hipStream_t stream = 0) {
+    template <class Grads>
+    float apply(Grads* grads, size_t embed_elems = 0, hipStream_t stream = 0) {
         optimizer_->set_embed_frozen(config_.freeze_embed && config_.freeze_in_plan);
+        optimizer_->set_fused_clip(config_.fused_clip);
+        optimizer_->set_zero_grads(config_.zero_grads);
         if (config_.freeze_embed && !config_.freeze_in_plan && embed_elems) {
             const size_t half_elems = grads->half_pool_bytes / sizeof(half);
             half* embed_grad = grads->half_pool + (half_elems - embed_elems);
@@ -47,7 +47,7 @@ public:
         float grad_norm = 0.0f;
         const bool clip = config_.max_grad_norm > 0.0f;
         if (clip) grad_norm = clip_grad_norm_(grads, config_.max_grad_norm, stream);
-        optimizer_->step(grads, stream, clip && config_.fused_clip, config_.zero_grads);
+        optimizer_->step(grads, stream);    // applies the scale itself after a fused clip_grad_norm_
         last_grad_norm_ = grad_norm;
         return grad_norm;
     }
@@ -79,6 +79,14 @@ private:
     OptimStepConfig config_;
     float last_grad_norm_ = 0.0f;
 };
+
+// Body for the reference's Trainer::clip_grad_norm_(Qwen3Gradients* grads, float max_norm) (trainer.h:323-352),
+// whose call sites (trainer.h:282, GRPO_trainer.h:511) then stay as they are:
+//     float clip_grad_norm_(Qwen3Gradients* grads, float max_norm) { return ::clip_grad_norm_(optimizer_, grads, max_norm); }
+template <class Grads>
+inline float clip_grad_norm_(AdamWOptimizer& optimizer, Grads* grads, float max_norm) {
+    return optimizer.clip_grad_norm_(grads, max_norm);
+}
 
 // The optimizer end of Trainer::train (include/training/trainer.h:183-225): per step set the scheduled
 // rate, obtain gradients (produce_grads(step) stands for the forward/backward passes and returns the
