@@ -197,74 +197,116 @@ class AdamWOptimizer:
         self.plan.adamw(self.step_params(), flags, _stream() if stream is None else stream)
 
     # --- optimizer state on disk (the reference's save_checkpoint is a stub, trainer.h:317-319) ----
-    CKPT_MAGIC = b"RLXOPT01"
+    # One format, shared with the C++ AdamWOptimizer (rl.cu_amd/host/training/optimizer.h): "RLXOPT02", int32
+    # step, 5 x float32 (lr, beta1, beta2, eps, weight_decay), int32 sections; per section uint16 name length,
+    # name, uint8 dtype (1 = FP32), int64 count, uint64 sum of the data's 32-bit words, data.  Sections, in this
+    # order, each over a whole pool (all FP16 tensors in list order, then all FP32 tensors, without the padding
+    # between tensors) and left out when empty: fp16.master (if kept), fp16.m, fp16.v, fp32.m, fp32.v.
+    CKPT_MAGIC = b"RLXOPT02"
+    CKPT_STAGE = 16 << 20            # elements per host staging buffer (64 MB)
+
+    def _state_sections(self):
+        """[(name, [tensor views in pool order], total count)] of this optimizer's state."""
+        st = self.store
+        idx16 = [i for i, s in enumerate(st.specs) if s.dtype == DTYPE_F16]
+        idx32 = [i for i, s in enumerate(st.specs) if s.dtype == DTYPE_F32]
+        out = []
+        for pool, idx, kinds in (("fp16", idx16, (("master",) if st.master is not None else ()) + ("m", "v")),
+                                 ("fp32", idx32, ("m", "v"))):
+            for which in kinds:
+                views = [st.state(i, which) for i in idx]
+                total = sum(v.numel() for v in views)
+                if total:
+                    out.append((pool + "." + which, views, total))
+        return out
+
+    def _stage_chunks(self, views):
+        for t in views:
+            for lo in range(0, t.numel(), self.CKPT_STAGE):
+                yield t[lo: lo + self.CKPT_STAGE]
 
     def save_state(self, path):
-        """Writes step counter, hyper-parameters and m, v (and master) of every tensor.
-        Layout: magic, int32 step, 5 x float32 (lr, beta1, beta2, eps, weight_decay), int32 sections, then per
-        section: uint16 name length, name, uint8 dtype (1 = FP32), int64 count, uint64 sum of the data's 32-bit
-        words, data."""
+        """Writes step counter, hyper-parameters and the pooled m, v (and master) sections."""
         import numpy as np
         import torch
         torch.cuda.synchronize()
-        st = self.store
-        secs = []
-        for i, s in enumerate(st.specs):
-            for which in ("m", "v") + (("master",) if (st.master is not None and s.dtype == DTYPE_F16) else ()):
-                secs.append((s.name + "." + which, st.state(i, which)))
+        secs = self._state_sections()
         tmp = path + ".tmp"
         with open(tmp, "wb") as f:
             f.write(self.CKPT_MAGIC)
             f.write(struct.pack("<i5fi", self.step_, self.lr, self.beta1, self.beta2, self.eps, self.weight_decay,
                                 len(secs)))
-            for name, t in secs:
-                a = t.detach().cpu().numpy()
+            for name, views, total in secs:
                 nb = name.encode()
                 f.write(struct.pack("<H", len(nb)) + nb)
-                f.write(struct.pack("<BqQ", 1, a.size, int(a.view(np.uint32).sum(dtype=np.uint64))))
-                f.write(a.tobytes())
+                f.write(struct.pack("<Bq", 1, total))
+                sum_at = f.tell()
+                f.write(struct.pack("<Q", 0))                  # patched once the data has passed
+                csum = 0
+                for part in self._stage_chunks(views):
+                    a = part.detach().cpu().numpy()
+                    csum = (csum + int(a.view(np.uint32).sum(dtype=np.uint64))) & 0xFFFFFFFFFFFFFFFF
+                    f.write(a.tobytes())
+                end = f.tell()
+                f.seek(sum_at)
+                f.write(struct.pack("<Q", csum))
+                f.seek(end)
         os.replace(tmp, path)
 
     def load_state(self, path):
-        """Restores what save_state wrote into this optimizer's store; the tensor list must be the same.
-        Raises ValueError on a foreign, truncated or corrupted file and leaves the state untouched then."""
+        """Restores what save_state (or the C++ class) wrote; the pools must have the same sizes.  The whole
+        file is checked first; a foreign, truncated, damaged or differently laid out file raises ValueError (the
+        message says which) and leaves the state untouched."""
         import numpy as np
         import torch
-        st = self.store
-        want = []
-        for i, s in enumerate(st.specs):
-            for which in ("m", "v") + (("master",) if (st.master is not None and s.dtype == DTYPE_F16) else ()):
-                want.append((s.name + "." + which, i, which, s.n))
-        loaded = []
+        secs = self._state_sections()
+        data_at = []
         with open(path, "rb") as f:
-            if f.read(8) != self.CKPT_MAGIC:
+            magic = f.read(8)
+            if magic == b"RLXOPT01":
+                raise ValueError("optimizer state in the older RLXOPT01 layout, which is no longer read: " + path)
+            if magic != self.CKPT_MAGIC:
                 raise ValueError("not an optimizer state file: " + path)
             head = f.read(28)
             if len(head) != 28:
-                raise ValueError("truncated optimizer state file")
+                raise ValueError("truncated optimizer state file (header)")
             step, lr, b1, b2, eps, wd, nsec = struct.unpack("<i5fi", head)
-            if nsec != len(want):
-                raise ValueError("optimizer state has %d sections, this optimizer needs %d" % (nsec, len(want)))
-            for name, i, which, n in want:
+            if step < 0 or not all(math.isfinite(x) for x in (lr, b1, b2, eps, wd)):
+                raise ValueError("optimizer state with a negative step or a hyper-parameter that is not finite")
+            if nsec != len(secs):
+                raise ValueError("optimizer state has %d sections, this optimizer has %d (different layout: master "
+                                 "copy or FP32 pool present on one side only)" % (nsec, len(secs)))
+            for name, views, total in secs:                    # pass 1: headers and checksums, nothing is changed
                 raw = f.read(2)
                 if len(raw) != 2:
-                    raise ValueError("truncated optimizer state file")
+                    raise ValueError("truncated optimizer state file (section header)")
                 (ln,) = struct.unpack("<H", raw)
-                got = f.read(ln).decode()
+                got = f.read(ln).decode(errors="replace")
                 meta = f.read(17)
                 if len(meta) != 17:
-                    raise ValueError("truncated optimizer state file")
-                dt, cnt, csum = struct.unpack("<BqQ", meta)
-                if got != name or dt != 1 or cnt != n:
-                    raise ValueError("section %r (%d) does not match tensor %r (%d)" % (got, cnt, name, n))
-                a = np.frombuffer(f.read(4 * n), dtype=np.float32)
-                if a.size != n:
-                    raise ValueError("truncated optimizer state file")
-                if int(a.view(np.uint32).sum(dtype=np.uint64)) != csum:
-                    raise ValueError("checksum mismatch in section " + name)
-                loaded.append((i, which, a))
-        for i, which, a in loaded:
-            st.state(i, which).copy_(torch.from_numpy(a.copy()))
+                    raise ValueError("truncated optimizer state file (section header)")
+                dt, cnt, want = struct.unpack("<BqQ", meta)
+                if got != name or dt != 1 or cnt != total:
+                    raise ValueError("section %r with %d values where this optimizer needs %r with %d (different "
+                                     "model or layout)" % (got, cnt, name, total))
+                data_at.append(f.tell())
+                csum, left = 0, total
+                while left:
+                    k = min(left, self.CKPT_STAGE)
+                    a = np.fromfile(f, dtype=np.uint32, count=k)
+                    if a.size != k:
+                        raise ValueError("truncated optimizer state file (data of %s)" % name)
+                    csum = (csum + int(a.sum(dtype=np.uint64))) & 0xFFFFFFFFFFFFFFFF
+                    left -= k
+                if csum != want:
+                    raise ValueError("damaged optimizer state file: checksum mismatch in section " + name)
+            if f.read(1):
+                raise ValueError("optimizer state file is longer than its sections")
+            for (name, views, total), at in zip(secs, data_at):     # pass 2: copy to the device
+                f.seek(at)
+                for part in self._stage_chunks(views):
+                    a = np.fromfile(f, dtype=np.float32, count=part.numel())
+                    part.copy_(torch.from_numpy(a))
         self.step_, self.lr, self.beta1, self.beta2, self.eps, self.weight_decay = step, lr, b1, b2, eps, wd
         torch.cuda.synchronize()
 

@@ -13,6 +13,8 @@
 // three launches (projections with decay, embedding and norm weights without), this issues
 // one multi-tensor launch with the same three groups.
 #pragma once
+#include <sys/types.h>
+
 #include <cassert>
 #include <cmath>
 #include <cstdint>
@@ -257,11 +259,15 @@ public:
         return total_norm;
     }
 
-    // Optimizer state on disk (the reference's save_checkpoint is a stub, trainer.h:317-319).
-    // File: "RLXOPT01", int32 step, 5 floats (lr, beta1, beta2, eps, weight_decay), int32 sections;
+    // Optimizer state on disk (the reference's save_checkpoint is a stub, trainer.h:317-319, so the format is
+    // this library's; rl.cu_amd/host.py reads and writes the same files).
+    // File: "RLXOPT02", int32 step, 5 floats (lr, beta1, beta2, eps, weight_decay), int32 sections;
     // per section: uint16 name length, name, uint8 dtype (1 = FP32), int64 count, uint64 sum of the
-    // data's 32-bit words, data.  Sections: fp16.master (if kept), fp16.m, fp16.v, fp32.m, fp32.v.
-    // Both return false (and print why) on failure; load_state leaves the state alone then.
+    // data's 32-bit words, data.  Sections, in this order, each over a whole pool (all FP16 tensors in pool
+    // order, then all FP32 tensors) and left out when empty: fp16.master (if kept), fp16.m, fp16.v, fp32.m,
+    // fp32.v.  Data moves through a 64 MB staging buffer, so the host never holds a whole pool.
+    // Both return false (and print why) on failure; load_state checks the whole file before it touches the
+    // state and leaves it alone if anything is wrong.
     bool save_state(const std::string& path) const {
         HIP_CHECK(hipDeviceSynchronize());
         const std::string tmp = path + ".tmp";
@@ -270,23 +276,30 @@ public:
         const std::vector<Section> secs = sections();
         const int32_t step = step_, nsec = (int32_t)secs.size();
         const float hyper[5] = {lr, beta1, beta2, eps, weight_decay};
-        bool ok = fwrite("RLXOPT01", 1, 8, f) == 8 && fwrite(&step, 4, 1, f) == 1 && fwrite(hyper, 4, 5, f) == 5 &&
+        bool ok = fwrite(kStateMagic, 1, 8, f) == 8 && fwrite(&step, 4, 1, f) == 1 && fwrite(hyper, 4, 5, f) == 5 &&
                   fwrite(&nsec, 4, 1, f) == 1;
-        std::vector<float> host;
+        std::vector<float> stage(stage_floats(secs));
         for (const Section& s : secs) {
-            host.resize(s.n);
-            HIP_CHECK(hipMemcpy(host.data(), s.dev, s.n * sizeof(float), hipMemcpyDeviceToHost));
+            if (!ok) break;
             const uint16_t len = (uint16_t)s.name.size();
             const uint8_t dtype = 1;
             const int64_t count = (int64_t)s.n;
-            const uint64_t sum = word_sum(host.data(), s.n);
-            ok = ok && fwrite(&len, 2, 1, f) == 1 && fwrite(s.name.data(), 1, len, f) == len &&
-                 fwrite(&dtype, 1, 1, f) == 1 && fwrite(&count, 8, 1, f) == 1 && fwrite(&sum, 8, 1, f) == 1 &&
-                 fwrite(host.data(), sizeof(float), s.n, f) == s.n;
+            uint64_t sum = 0;
+            ok = fwrite(&len, 2, 1, f) == 1 && fwrite(s.name.data(), 1, len, f) == len &&
+                 fwrite(&dtype, 1, 1, f) == 1 && fwrite(&count, 8, 1, f) == 1;
+            const off_t sum_at = ftello(f);
+            ok = ok && sum_at >= 0 && fwrite(&sum, 8, 1, f) == 1;      // patched below, once the data has passed
+            for (size_t done = 0; ok && done < s.n; done += stage.size()) {
+                const size_t k = s.n - done < stage.size() ? s.n - done : stage.size();
+                HIP_CHECK(hipMemcpy(stage.data(), s.dev + done, k * sizeof(float), hipMemcpyDeviceToHost));
+                sum += word_sum(stage.data(), k);
+                ok = fwrite(stage.data(), sizeof(float), k, f) == k;
+            }
+            ok = ok && fseeko(f, sum_at, SEEK_SET) == 0 && fwrite(&sum, 8, 1, f) == 1 && fseeko(f, 0, SEEK_END) == 0;
         }
         ok = (fclose(f) == 0) && ok;
         if (ok) ok = rename(tmp.c_str(), path.c_str()) == 0;
-        if (!ok) fprintf(stderr, "[AdamW] writing %s failed\n", path.c_str());
+        if (!ok) { fprintf(stderr, "[AdamW] writing %s failed\n", path.c_str()); remove(tmp.c_str()); }
         return ok;
     }
 
@@ -294,30 +307,67 @@ public:
         FILE* f = fopen(path.c_str(), "rb");
         if (!f) { fprintf(stderr, "[AdamW] cannot read %s\n", path.c_str()); return false; }
         const std::vector<Section> secs = sections();
+        std::string why;
         char magic[8];
         int32_t step = 0, nsec = 0;
-        float hyper[5];
-        bool ok = fread(magic, 1, 8, f) == 8 && memcmp(magic, "RLXOPT01", 8) == 0 && fread(&step, 4, 1, f) == 1 &&
-                  fread(hyper, 4, 5, f) == 5 && fread(&nsec, 4, 1, f) == 1 && nsec == (int32_t)secs.size();
-        std::vector<std::vector<float>> data(secs.size());
-        for (size_t i = 0; ok && i < secs.size(); i++) {
+        float hyper[5] = {};
+        if (fread(magic, 1, 8, f) != 8) why = "shorter than a header";
+        else if (memcmp(magic, "RLXOPT01", 8) == 0) why = "written in the older RLXOPT01 layout, which is no longer read";
+        else if (memcmp(magic, kStateMagic, 8) != 0) why = "not an optimizer state file";
+        else if (fread(&step, 4, 1, f) != 1 || fread(hyper, 4, 5, f) != 5 || fread(&nsec, 4, 1, f) != 1) why = "truncated header";
+        else if (step < 0) why = "negative step counter";
+        else if (nsec != (int32_t)secs.size())
+            why = "holds " + std::to_string(nsec) + " sections, this optimizer has " + std::to_string(secs.size()) +
+                  " (different layout: master copy or FP32 pool present on one side only)";
+        for (int k = 0; why.empty() && k < 5; k++)
+            if (!std::isfinite(hyper[k])) why = "hyper-parameter that is not finite";
+        // pass 1: every section header must match and every checksum must hold, before anything is changed
+        std::vector<float> stage(why.empty() ? stage_floats(secs) : 0);
+        std::vector<off_t> data_at(secs.size(), 0);
+        for (size_t i = 0; why.empty() && i < secs.size(); i++) {
             uint16_t len = 0;
             uint8_t dtype = 0;
             int64_t count = 0;
-            uint64_t sum = 0;
+            uint64_t want = 0, sum = 0;
             char name[256];
-            ok = fread(&len, 2, 1, f) == 1 && len < sizeof(name) && fread(name, 1, len, f) == len &&
-                 fread(&dtype, 1, 1, f) == 1 && fread(&count, 8, 1, f) == 1 && fread(&sum, 8, 1, f) == 1 &&
-                 std::string(name, len) == secs[i].name && dtype == 1 && count == (int64_t)secs[i].n;
-            if (!ok) break;
-            data[i].resize(secs[i].n);
-            ok = fread(data[i].data(), sizeof(float), secs[i].n, f) == secs[i].n &&
-                 word_sum(data[i].data(), secs[i].n) == sum;
+            if (fread(&len, 2, 1, f) != 1 || len >= sizeof(name) || fread(name, 1, len, f) != len ||
+                fread(&dtype, 1, 1, f) != 1 || fread(&count, 8, 1, f) != 1 || fread(&want, 8, 1, f) != 1) {
+                why = "truncated in the header of section " + std::to_string(i);
+            } else if (std::string(name, len) != secs[i].name || dtype != 1 || count != (int64_t)secs[i].n) {
+                why = "section " + std::to_string(i) + " is '" + std::string(name, len) + "' with " + std::to_string(count) +
+                      " values, this optimizer needs '" + secs[i].name + "' with " + std::to_string(secs[i].n) +
+                      " (different model or layout)";
+            } else {
+                data_at[i] = ftello(f);
+                for (size_t done = 0; why.empty() && done < secs[i].n; done += stage.size()) {
+                    const size_t k = secs[i].n - done < stage.size() ? secs[i].n - done : stage.size();
+                    if (fread(stage.data(), sizeof(float), k, f) != k) why = "truncated in the data of section '" + secs[i].name + "'";
+                    else sum += word_sum(stage.data(), k);
+                }
+                if (why.empty() && sum != want) why = "damaged: checksum of section '" + secs[i].name + "' does not match";
+            }
+        }
+        if (why.empty() && fgetc(f) != EOF) why = "longer than its sections";
+        if (!why.empty()) {
+            fclose(f);
+            fprintf(stderr, "[AdamW] %s: %s\n", path.c_str(), why.c_str());
+            return false;
+        }
+        // pass 2: copy to the device
+        bool ok = true;
+        for (size_t i = 0; ok && i < secs.size(); i++) {
+            ok = fseeko(f, data_at[i], SEEK_SET) == 0;
+            for (size_t done = 0; ok && done < secs[i].n; done += stage.size()) {
+                const size_t k = secs[i].n - done < stage.size() ? secs[i].n - done : stage.size();
+                ok = fread(stage.data(), sizeof(float), k, f) == k;
+                if (ok) HIP_CHECK(hipMemcpy(secs[i].dev + done, stage.data(), k * sizeof(float), hipMemcpyHostToDevice));
+            }
         }
         fclose(f);
-        if (!ok) { fprintf(stderr, "[AdamW] %s is not a matching, intact optimizer state\n", path.c_str()); return false; }
-        for (size_t i = 0; i < secs.size(); i++)
-            HIP_CHECK(hipMemcpy(secs[i].dev, data[i].data(), secs[i].n * sizeof(float), hipMemcpyHostToDevice));
+        if (!ok) {      // the file changed under us between the passes: the state is now partly overwritten
+            fprintf(stderr, "[AdamW] %s: read error while loading; the optimizer state is incomplete\n", path.c_str());
+            exit(1);
+        }
         step_ = step;
         lr = hyper[0]; beta1 = hyper[1]; beta2 = hyper[2]; eps = hyper[3]; weight_decay = hyper[4];
         return true;
@@ -394,6 +444,13 @@ private:
         if (n16_) { s.push_back({"fp16.m", fp16_m_, n16_}); s.push_back({"fp16.v", fp16_v_, n16_}); }
         if (n32_) { s.push_back({"fp32.m", fp32_m_, n32_}); s.push_back({"fp32.v", fp32_v_, n32_}); }
         return s;
+    }
+    static constexpr const char* kStateMagic = "RLXOPT02";
+    static constexpr size_t kStageFloats = (size_t)16 << 20;         // 64 MB between the device and the file
+    static size_t stage_floats(const std::vector<Section>& secs) {
+        size_t most = 1;
+        for (const Section& s : secs) most = s.n > most ? s.n : most;
+        return most < kStageFloats ? most : kStageFloats;
     }
     static uint64_t word_sum(const float* p, size_t n) {
         uint64_t acc = 0;

@@ -77,6 +77,161 @@ def test_checkpoint_rejects_bad_files(L, host, torch_gpu, tmp_path):
         other.load_state(path)
 
 
+# --- one optimizer-state format for the C++ class and the Python class, checked against the oracle -----------
+XCFG = dict(vocab=512, hidden=128, inter=256, layers=2, q_heads=2, kv_heads=1, head_dim=128, tied=True)
+XTAIL, XLR, XMAX, XSTD = 148, 1e-3, 0.5, 5e-3          # the constants of tests/cpp/ckpt_tool.cpp
+XTOOL = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "ckpt_tool.bin")
+
+
+class PoolWorld:
+    """Python twin of the model in ckpt_tool.cpp: the same pools (every tensor a multiple of 128 elements, so
+    the store's pools have no padding), the same seeds, a workspace tail that only takes part in the norm."""
+
+    def __init__(self, L, host, torch, master=True):
+        self.specs = L.qwen3_tensor_list(XCFG, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
+        self.n16 = sum(s.n for s in self.specs if s.dtype == L.DTYPE_F16)
+        self.n32 = sum(s.n for s in self.specs if s.dtype == L.DTYPE_F32)
+        self.proj_n = self.n16 - XCFG["vocab"] * XCFG["hidden"]
+        self.st = host.ParamStore(self.specs, master=master)
+        assert self.st.p16.numel() == self.n16 and self.st.p32.numel() == self.n32
+        self.tail = torch.zeros(XTAIL, dtype=torch.float32, device="cuda:0")
+        self.host, self.L = host, L
+
+    def optimizer(self):
+        return self.host.AdamWOptimizer(self.st, lr=XLR, extra_grad_only=(self.tail,))
+
+    def seed_weights(self, B):
+        B.fill_f16(self.st.p16.data_ptr(), self.n16, 71, 0.0, 0.02)
+        B.fill_f32(self.st.p32.data_ptr(), self.n32, 72, 1.0, 0.05)
+        self.st.init_master()
+
+    def step(self, B, opt, s):
+        B.fill_f16(self.st.g16.data_ptr(), self.n16, 5000 + 2 * s, 0.0, XSTD)
+        B.fill_f32(self.st.g32.data_ptr(), self.n32, 5001 + 2 * s, 0.0, XSTD)
+        B.fill_f32(self.tail.data_ptr(), XTAIL, 5001 + 2 * s, 0.0, XSTD, first=self.n32)
+        return self.host.training_step(opt, XMAX, fused_clip=False)
+
+    def norm_groups(self, g16, g32):
+        """The gradient arrays in the order of this optimizer's plan: tensor by tensor, then the tail."""
+        out, o16, o32 = [], 0, 0
+        for s in self.specs:
+            if s.dtype == self.L.DTYPE_F16:
+                out.append(g16[o16: o16 + s.n])
+                o16 += s.n
+            else:
+                out.append(g32[o32: o32 + s.n])
+                o32 += s.n
+        return out + [g32[self.n32:]]
+
+
+class OracleReplay:
+    """The reference's order of operations on the host, from the seeded start: norm (added up in the order of
+    the plan that ran the step) -> scale in place if norm > max -> three-group step."""
+
+    def __init__(self, O, w):
+        import numpy as np
+        self.O, self.w, self.np = O, w, np
+        self.w16 = O.fill_f16(w.n16, 71, 0.0, 0.02)
+        self.w32 = O.fill_f32(w.n32, 72, 1.0, 0.05)
+        self.master = O.h2f(self.w16)
+        self.m16, self.v16 = np.zeros(w.n16, np.float32), np.zeros(w.n16, np.float32)
+        self.m32, self.v32 = np.zeros(w.n32, np.float32), np.zeros(w.n32, np.float32)
+        self.step_ = 0
+        self.norms = []
+
+    def step(self, s, cxx_order, chunk):
+        O, w, np = self.O, self.w, self.np
+        g16 = O.fill_f16(w.n16, 5000 + 2 * s, 0.0, XSTD)
+        g32 = O.fill_f32(w.n32 + XTAIL, 5001 + 2 * s, 0.0, XSTD)
+        groups = [g16[:w.proj_n], g16[w.proj_n:], g32[:w.n32], g32[w.n32:]] if cxx_order else w.norm_groups(g16, g32)
+        ssq, _ = O.sumsq_mirror(groups, chunk)
+        scale, norm = O.clip_scale(ssq, XMAX)
+        assert norm > XMAX
+        O.scale_half(g16, scale)
+        O.scale_float(g32, scale)
+        self.norms.append(norm)
+        self.step_ = O.optimizer_step(self.master, self.w16, g16, self.m16, self.v16, w.proj_n, self.w32,
+                                      np.ascontiguousarray(g32[:w.n32]), self.m32, self.v32, XLR, 0.9, 0.999, 1e-8,
+                                      0.01, self.step_)
+
+
+def run_tool(*args):
+    import subprocess
+    if not os.path.exists(XTOOL):
+        subprocess.run(["make", "-C", os.path.dirname(XTOOL), "-s"], check=True)
+    return subprocess.run([XTOOL] + [str(a) for a in args], capture_output=True, text=True, timeout=100)
+
+
+def test_state_saved_by_cxx_loads_in_python_and_continues_as_the_oracle(O, B, L, host, torch_gpu, tmp_path):
+    """ckpt_tool (C++ AdamWOptimizer) takes 3 steps and saves; the Python AdamWOptimizer loads that file and
+    takes steps 4 and 5; weights, master copy and moments equal the oracle's five steps from the seeded start."""
+    import numpy as np
+    from util import bits
+    torch = torch_gpu
+    res = run_tool("save", tmp_path, 3)
+    assert res.returncode == 0, res.stdout + res.stderr
+    w = PoolWorld(L, host, torch)
+    w.st.p16.copy_(torch.from_numpy(np.fromfile(tmp_path / "w16.bin", dtype=np.int16)).view(torch.float16))
+    w.st.p32.copy_(torch.from_numpy(np.fromfile(tmp_path / "w32.bin", dtype=np.float32)))
+    opt = w.optimizer()
+    opt.load_state(str(tmp_path / "opt.state"))
+    assert opt.get_step() == 3
+    got_norms = [w.step(B, opt, s) for s in (4, 5)]
+    torch.cuda.synchronize()
+    rep = OracleReplay(O, w)
+    for s in (1, 2, 3):
+        rep.step(s, cxx_order=True, chunk=8192)
+    cxx_norms = [float(line.split()[3]) for line in res.stdout.splitlines() if line.startswith("step ")]
+    assert [np.float32(x) for x in cxx_norms] == [np.float32(x) for x in rep.norms]
+    for s in (4, 5):
+        rep.step(s, cxx_order=False, chunk=opt.plan.chunk_elems)
+    assert [np.float32(x) for x in got_norms] == [np.float32(x) for x in rep.norms[3:]]
+    st = w.st
+    assert np.array_equal(bits(st.p16), rep.w16) and np.array_equal(bits(st.p32).view(np.uint32), rep.w32.view(np.uint32))
+    assert np.array_equal(bits(st.master[:w.n16]).view(np.uint32), rep.master.view(np.uint32))
+    for got, want in ((st.m[:w.n16], rep.m16), (st.v[:w.n16], rep.v16), (st.m[w.n16:], rep.m32), (st.v[w.n16:], rep.v32)):
+        assert np.array_equal(bits(got).view(np.uint32), want.view(np.uint32))
+    # the same file does not fit an optimizer without a master copy, and the error says so
+    other = PoolWorld(L, host, torch, master=False).optimizer()
+    with pytest.raises(ValueError, match="different layout"):
+        other.load_state(str(tmp_path / "opt.state"))
+
+
+def test_state_saved_by_python_loads_in_cxx_and_continues_as_the_oracle(O, B, L, host, torch_gpu, tmp_path):
+    """The Python AdamWOptimizer takes 3 steps and saves; ckpt_tool loads that file into the C++ class and takes
+    steps 4 and 5; what it ends with equals the oracle's five steps.  A damaged copy of the file is refused."""
+    import numpy as np
+    from util import bits
+    torch = torch_gpu
+    w = PoolWorld(L, host, torch)
+    w.seed_weights(B)
+    opt = w.optimizer()
+    for s in (1, 2, 3):
+        w.step(B, opt, s)
+    torch.cuda.synchronize()
+    opt.save_state(str(tmp_path / "opt.state"))
+    bits(w.st.p16).tofile(tmp_path / "w16.bin")
+    bits(w.st.p32).tofile(tmp_path / "w32.bin")
+    res = run_tool("load", tmp_path, 3, 2)
+    assert res.returncode == 0, res.stdout + res.stderr
+    rep = OracleReplay(O, w)
+    for s in (1, 2, 3):
+        rep.step(s, cxx_order=False, chunk=opt.plan.chunk_elems)
+    for s in (4, 5):
+        rep.step(s, cxx_order=True, chunk=8192)
+    cxx_norms = [float(line.split()[3]) for line in res.stdout.splitlines() if line.startswith("step ")]
+    assert [np.float32(x) for x in cxx_norms] == [np.float32(x) for x in rep.norms[3:]]
+    assert np.array_equal(np.fromfile(tmp_path / "out_w16.bin", dtype=np.uint16), rep.w16)
+    for name, want in (("w32", rep.w32), ("master", rep.master), ("m16", rep.m16), ("v16", rep.v16),
+                       ("m32", rep.m32), ("v32", rep.v32)):
+        assert np.array_equal(np.fromfile(tmp_path / ("out_%s.bin" % name), dtype=np.uint32), want.view(np.uint32)), name
+    # a flipped data bit, a cut file and a foreign file are refused by the C++ loader (exit code 3)
+    good = open(tmp_path / "opt.state", "rb").read()
+    for blob in (good[:-5] + bytes([good[-5] ^ 0x40]) + good[-4:], good[: len(good) // 2], b"RLXOPT01" + good[8:]):
+        open(tmp_path / "opt.state", "wb").write(blob)
+        assert run_tool("load", tmp_path, 3, 1).returncode == 3
+
+
 def test_train_loop_logs_jsonl(L, host, torch_gpu, tmp_path, capsys):
     """Cosine schedule with warm-up drives set_lr; every second step one JSON line with the window means of
     loss, lr, grad_norm, step_ms, tok_per_sec (the keys of include/training/trainer.h:208-212)."""
