@@ -1,18 +1,23 @@
 #!/usr/bin/env python3
 """Benchmark of the AdamW step on one MI355X.
 
-Workload (N=1): the Qwen3-0.6B parameter set as a 310-tensor list, FP16 parameters and
+Headline workload (N=1): the Qwen3-0.6B parameter set as a 310-tensor list, FP16 parameters and
 gradients, FP32 moments, no master copy; moments pre-populated by 99 seeded steps; timed steps
 are steps 100, 101, ... over resident inputs: one multi-tensor update launch each (22 bytes per
 parameter: read p, g, m, v; write p, m, v).  The same list with the norm + fused-clip step is
 timed too and reported under "clip_step".
 
+The default run also measures the other configurations (one flat tensor of 1,048,576 parameters, the
+4,096-tensor ragged list beside one flat tensor of the same element count, the Qwen3-8B list, and
+Qwen3-0.6B in the reference's 28-byte layout with an FP32 master copy) and reports them under "configs":
+update, norm, norm + fused-clip update, each in ms and GB/s (seeded state, no oracle replay: the GPU tests
+hold the parity of these configurations).  --configs none skips them (short profiler runs).
+
 Prints ONE JSON line.  The CPU oracle is used here only as the checker of a sample and as the
 timed CPU baseline.
 
---workload selects one of the other configurations instead (flat-1m, qwen3-0.6b-master, ragged,
-qwen3-8b): the same kind of line with fewer legs (update, norm, norm + fused-clip update; seeded
-state, no oracle replay: the GPU tests hold the parity of these configurations).
+--workload selects one of the other configurations as the line's subject instead (flat-1m,
+qwen3-0.6b-master, ragged, qwen3-8b): the same kind of line with fewer legs.
 """
 import argparse
 import importlib
@@ -29,46 +34,80 @@ HBM_PEAK_GBPS = 8000.0
 BYTES_UPDATE = 22          # per parameter: R p2 g2 m4 v4, W p2 m4 v4
 BYTES_NORM = 2             # per parameter: R g2
 SEED_P, SEED_G = 0x5EED0001, 0x6EAD0001
+STORAGE = "fp16 params and grads, fp32 moments; arithmetic in fp32"
+SECONDARY = ("flat-1m", "ragged", "qwen3-0.6b-master", "qwen3-8b")
 
 
 def log(*a):
     print(*a, file=sys.stderr, flush=True)
 
 
-def cpu_baseline(O, host, sample, hyper, step, seconds=8.0):
-    """The oracle's threaded FP16 step (norm off) on a slice of the same workload, repeated
-    until about `seconds` of wall time have passed."""
-    import numpy as np
+def host_cpus():
+    """What this process may use: logical CPUs, the affinity mask, and the cgroup's quota if there is one."""
+    info = {"nproc": os.cpu_count() or 1}
+    try:
+        info["affinity"] = len(os.sched_getaffinity(0))
+    except (AttributeError, OSError):
+        info["affinity"] = info["nproc"]
+    try:
+        quota, period = open("/sys/fs/cgroup/cpu.max").read().split()
+        info["cgroup_cpus"] = None if quota == "max" else float(quota) / float(period)
+    except (OSError, ValueError):
+        info["cgroup_cpus"] = None
+    return info
+
+
+def cpu_baseline(O, host, sample, g_clip, hyper, step, seconds=5.0):
+    """The oracle's threaded FP16 step on a slice of the same workload, on the host's cores: the update alone
+    (the configuration of the headline), and norm + clip + update with the larger gradients of the clip
+    configuration (FP64 sum of squares, sqrt, scale = max/(norm+1e-6f) iff norm > max, then the update with
+    the scaled and re-rounded gradients).  Each leg is repeated until about `seconds` of wall time have
+    passed, with 16 threads (the CPU share of a one-GPU box) and with every core the process may use."""
     p, g, m, v = sample
-    threads = min(os.cpu_count() or 1, int(os.environ.get("OMP_NUM_THREADS", "16") or 16), 16)
+    cpus = host_cpus()
+    t16 = min(16, cpus["affinity"])
+    t_all = cpus["affinity"]
     bc1, bc2 = host.bias_correction(hyper["beta1"], step), host.bias_correction(hyper["beta2"], step)
     args = (hyper["lr"], hyper["beta1"], hyper["beta2"], hyper["eps"], hyper["wd"], bc1, bc2)
-    O.step_fp16_threaded(None, p, g, m, v, *args, 0.0, threads)          # touch pages, warm caches
-    reps, t0 = 0, time.perf_counter()
-    while True:
-        O.step_fp16_threaded(None, p, g, m, v, *args, 0.0, threads)
-        reps += 1
-        el = time.perf_counter() - t0
-        if el >= seconds or reps >= 200:
-            break
-    # one thread, on the first 4 Mi parameters of the sample
-    n1 = min(p.size, 4 * 1024 * 1024)
-    one = [a[:n1].copy() for a in (p, g, m, v)]
-    O.step_fp16_threaded(None, *one, *args, 0.0, 1)
-    r1, t1 = 0, time.perf_counter()
-    while time.perf_counter() - t1 < 2.0:
-        O.step_fp16_threaded(None, *one, *args, 0.0, 1)
-        r1 += 1
-    single = n1 * r1 / (time.perf_counter() - t1)
-    return {"value": p.size * reps / el, "unit": "params/s", "cores": threads, "kind": "port",
-            "single_thread_value": single,
-            "sample": "%d-parameter slice of embed_tokens (p, g, m, v after 99 steps), %d repeated steps, "
-                      "%.1f s wall; oracle's threaded AdamW loop, gcc -O3, no FMA contraction" % (p.size, reps, el),
-            "gbps": BYTES_UPDATE * p.size * reps / el / 1e9}
+
+    def rate(arrays, max_norm, threads, budget):
+        O.step_fp16_threaded(None, *arrays, *args, max_norm, threads)          # touch pages, warm caches
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            O.step_fp16_threaded(None, *arrays, *args, max_norm, threads)
+            reps += 1
+            el = time.perf_counter() - t0
+            if el >= budget or reps >= 200:
+                break
+        return arrays[0].size * reps / el, reps, el
+
+    out = {"unit": "params/s", "kind": "port", "nproc": cpus["nproc"], "affinity": cpus["affinity"],
+           "cgroup_cpus": cpus["cgroup_cpus"], "threads": t16, "threads_all_cores": t_all}
+    upd, reps, el = rate((p, g, m, v), 0.0, t16, seconds)
+    out["update"] = upd
+    out["value"] = upd
+    out["cores"] = t16
+    out["gbps"] = BYTES_UPDATE * upd / 1e9
+    clip_arrays = (p.copy(), g_clip, m.copy(), v.copy())
+    out["norm_clip_update"], reps_c, el_c = rate(clip_arrays, 1.0, t16, seconds)
+    if t_all != t16:
+        out["update_all_cores"], _, _ = rate((p, g, m, v), 0.0, t_all, seconds * 0.6)
+        out["norm_clip_update_all_cores"], _, _ = rate(clip_arrays, 1.0, t_all, seconds * 0.6)
+    else:
+        out["update_all_cores"], out["norm_clip_update_all_cores"] = out["update"], out["norm_clip_update"]
+    n1 = min(p.size, 4 * 1024 * 1024)                                # one thread, first 4 Mi parameters
+    out["single_thread"], _, _ = rate(tuple(a[:n1].copy() for a in (p, g, m, v)), 0.0, 1, 2.0)
+    out["single_thread_value"] = out["single_thread"]
+    out["sample"] = ("%d-parameter slice of embed_tokens of the Qwen3-0.6B list (p, m, v after 99 steps; g of step 100 "
+                     "for the update leg, g~N(0,5e-3) with max_norm 1.0 for the norm+clip+update leg); %d and %d "
+                     "repeated steps in %.1f and %.1f s; oracle's threaded AdamW loop, gcc -O3, no FMA contraction, "
+                     "static contiguous split over the threads" % (p.size, reps, reps_c, el, el_c))
+    return out
 
 
 def time_events(fn, warmup, steps):
-    """ms per call: `steps` calls back to back between two events on torch's current stream."""
+    """ms per call: `steps` calls back to back between two events on torch's current stream (the stream
+    every kernel here is launched on)."""
     import torch
     for _ in range(warmup):
         fn()
@@ -82,11 +121,11 @@ def time_events(fn, warmup, steps):
     return a.elapsed_time(b) / steps
 
 
-def other_workload(args, pkg, host):
-    """Update, norm and norm + fused-clip update of one of the secondary configurations."""
+def measure_workload(name, pkg, host, steps, warmup, chunk=0):
+    """Update, norm and norm + fused-clip update of one of the secondary configurations, from seeded state."""
     import torch
     B, L = pkg.binding, pkg.layout
-    name, master, extra = args.workload, False, {}
+    master = False
     if name == "flat-1m":
         specs = [L.TensorSpec("flat", 1 << 20, L.DTYPE_F16, 0, 0)]
         p_std, g_std, what = 0.02, 1e-3, "one flat tensor of 1,048,576 FP16 parameters (22 MB: cache-resident)"
@@ -103,6 +142,8 @@ def other_workload(args, pkg, host):
     else:
         raise SystemExit("unknown workload " + name)
     N = L.total_elements(specs)
+    if N < (1 << 26):         # cache-resident: launches of a few microseconds need many repetitions to time
+        steps, warmup = max(steps, 400), max(warmup, 50)
     st = host.ParamStore(specs, "cuda:0", master=master)
     st.fill("p", SEED_P, 1.0 if name == "ragged" else 0.0, p_std)
     st.fill("g", SEED_G, 0.0, g_std)
@@ -110,44 +151,69 @@ def other_workload(args, pkg, host):
     st.fill("v", SEED_P + 2, 1e-8, 1e-8, flags=B.FILL_ABS)
     if master:
         st.init_master()
-    opt = host.AdamWOptimizer(st, lr=1e-5, chunk_elems=args.chunk)
+    opt = host.AdamWOptimizer(st, lr=1e-5, chunk_elems=chunk)
     opt.step_ = 999
     stream = torch.cuda.current_stream().cuda_stream
     bpp = 28 if master else BYTES_UPDATE
-    steps, warm = args.steps, args.warmup
-    upd = time_events(lambda: opt.step(), warm, steps)
-    nrm = time_events(lambda: opt.plan.grad_norm(1.0, stream), warm, steps)
+    upd = time_events(lambda: opt.step(), warmup, steps)
+    nrm = time_events(lambda: opt.plan.grad_norm(1.0, stream), warmup, steps)
 
     def clip_step():
         opt.plan.grad_norm(1.0, stream)
         opt.step(fused_clip=True)
 
-    both = time_events(clip_step, warm, steps)
+    both = time_events(clip_step, warmup, steps)
     norm, scale, _ = opt.plan.norm_read(stream)
     scale_ms = time_events(lambda: opt.plan.scale_grads(stream), 1, 5)   # shrinks the gradients: last leg
-    if name == "ragged":      # against one flat tensor of the same element count
-        flat = host.ParamStore([L.TensorSpec("flat", N, L.DTYPE_F16, 0, 0)], "cuda:0")
-        fopt = host.AdamWOptimizer(flat, lr=1e-5)
-        extra["flat_tensor_same_count_ms"] = time_events(lambda: fopt.step(), warm, steps)
-    gbps = bpp * N / (upd * 1e-3) / 1e9
     out = {
-        "metric": "AdamW params/sec, %s step" % name, "value": N / (upd * 1e-3), "unit": "params/s",
-        "n_gpus": 1, "steps": steps, "warmup": warm, "ms_per_step": upd, "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": what, "params": N, "tensors": len(specs), "bytes_per_param": bpp,
-                   "chunk_elems": opt.plan.chunk_elems, "chunks": opt.plan.num_chunks,
-                   "update_variant": B.get_tuning("update_variant")},
-        "roofline": {"bound": "hbm", "achieved": gbps, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": gbps / HBM_PEAK_GBPS, "traffic": None, "kernel_ms": upd,
-                     "algorithmic_bytes_per_launch": bpp * N},
-        "cpu_baseline": None,
+        "workload": what, "params": N, "tensors": len(specs), "bytes_per_param": bpp,
+        "chunk_elems": opt.plan.chunk_elems, "chunks": opt.plan.num_chunks,
+        "update_ms": upd, "update_gbps": bpp * N / (upd * 1e-3) / 1e9, "params_per_s": N / (upd * 1e-3),
         "norm_ms": nrm, "norm_gbps": BYTES_NORM * N / (nrm * 1e-3) / 1e9,
-        "clip_step": {"ms_per_step": both, "achieved_gbps": (bpp + BYTES_NORM) * N / (both * 1e-3) / 1e9,
-                      "grad_norm": norm, "clip_scale": scale, "scale_pass_ms": scale_ms,
-                      "unfused_ms_per_step": both + scale_ms},
+        "clip_step_ms": both, "clip_step_gbps": (bpp + BYTES_NORM) * N / (both * 1e-3) / 1e9,
+        "grad_norm": norm, "clip_scale": scale, "scale_pass_ms": scale_ms, "unfused_clip_step_ms": both + scale_ms,
     }
-    out.update(extra)
-    print(json.dumps(out), flush=True)
+    out["update_frac_of_peak"] = out["update_gbps"] / HBM_PEAK_GBPS
+    out["clip_step_frac_of_peak"] = out["clip_step_gbps"] / HBM_PEAK_GBPS
+    if name == "ragged":      # against one flat tensor of the same element count
+        del opt, st
+        flat = host.ParamStore([L.TensorSpec("flat", N, L.DTYPE_F16, 0, 0)], "cuda:0")
+        flat.fill("p", SEED_P, 1.0, p_std)
+        flat.fill("g", SEED_G, 0.0, g_std)
+        fopt = host.AdamWOptimizer(flat, lr=1e-5)
+        fopt.step_ = 999
+        out["flat_update_ms"] = time_events(lambda: fopt.step(), warmup, steps)
+        out["flat_norm_ms"] = time_events(lambda: fopt.plan.grad_norm(1.0, stream), warmup, steps)
+
+        def flat_clip_step():
+            fopt.plan.grad_norm(1.0, stream)
+            fopt.step(fused_clip=True)
+
+        out["flat_clip_step_ms"] = time_events(flat_clip_step, warmup, steps)
+        out["update_vs_flat"] = upd / out["flat_update_ms"]
+        out["norm_vs_flat"] = nrm / out["flat_norm_ms"]
+        out["clip_step_vs_flat"] = both / out["flat_clip_step_ms"]
+        del fopt, flat
+    return out
+
+
+def workload_line(name, w, steps, warmup, B):
+    """The bench line of a secondary configuration (--workload)."""
+    variant = B.get_tuning("update_variant")
+    return {
+        "metric": "AdamW params/sec, %s step" % name, "value": w["params_per_s"], "unit": "params/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup, "ms_per_step": w["update_ms"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "storage": STORAGE, "data": "synthetic",
+        "config": {"workload": w["workload"], "params": w["params"], "tensors": w["tensors"],
+                   "bytes_per_param": w["bytes_per_param"], "chunk_elems": w["chunk_elems"], "chunks": w["chunks"],
+                   "update_variant": variant},
+        "roofline": {"bound": "hbm", "achieved": w["update_gbps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": w["update_gbps"] / HBM_PEAK_GBPS, "traffic": None, "traffic_source": None,
+                     "kernel": B.update_variant_name(variant), "kernel_ms": w["update_ms"],
+                     "algorithmic_bytes_per_launch": w["bytes_per_param"] * w["params"]},
+        "cpu_baseline": None,
+        "measured": {k: v for k, v in w.items() if k not in ("workload", "params", "tensors")},
+    }
 
 
 def main():
@@ -157,9 +223,12 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="qwen3-0.6b",
                     help="qwen3-0.6b (default, the headline), flat-1m, qwen3-0.6b-master, ragged, qwen3-8b")
+    ap.add_argument("--configs", default="all",
+                    help="with the headline workload: 'all' (default) also measures the other configurations and "
+                         "reports them under \"configs\"; 'none' skips them; or a comma-separated subset")
     ap.add_argument("--chunk", type=int, default=0, help="chunk_elems of the plan (0 = automatic)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--variant", type=int, default=None, help="update kernel tile shape (tuning)")
+    ap.add_argument("--variant", type=int, default=None, help="update kernel form (tuning key update_variant)")
     ap.add_argument("--quick-setup", action="store_true",
                     help="seed the moments directly instead of running 99 steps (short profiler runs: few "
                          "dispatches); the parity sample then covers one step")
@@ -183,7 +252,8 @@ def main():
     if args.variant is not None:
         B.set_tuning("update_variant", args.variant)
     if args.workload != "qwen3-0.6b":
-        other_workload(args, pkg, host)
+        w = measure_workload(args.workload, pkg, host, args.steps, args.warmup, args.chunk)
+        print(json.dumps(workload_line(args.workload, w, args.steps, args.warmup, B)), flush=True)
         return
 
     hyper = dict(lr=1e-5, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01)
@@ -265,9 +335,14 @@ def main():
     kernel_ms = ev_ms
     achieved = BYTES_UPDATE * N / (kernel_ms * 1e-3) / 1e9
 
+    # ---- CPU baseline sample: state of the headline configuration (before the clip leg moves it on) ----
+    n_s = 32 * 1024 * 1024
+    sample = None if args.no_cpu else tuple(grab(k, emb, 0, n_s) for k in ("p", "g", "m", "v"))
+
     # ---- timed: norm + clip scale + fused update (configs[2]); larger gradients so that clipping is active ----
     st.fill("g", SEED_G + 1000, 0.0, 5e-3)
     stream = torch.cuda.current_stream().cuda_stream
+    g_clip = None if args.no_cpu else grab("g", emb, 0, n_s)
 
     def clip_step():
         opt.plan.grad_norm(1.0, stream)
@@ -275,64 +350,91 @@ def main():
 
     cwall, cev_ms, cper = run(clip_step, max(2, args.warmup // 2), max(5, args.steps // 2))
     norm, scale, _ = opt.plan.norm_read(stream)
+    norm_ms = time_events(lambda: opt.plan.grad_norm(1.0, stream), 3, 20)
     clip = {"ms_per_step": cev_ms, "params_per_s": N / (cev_ms * 1e-3),
             "achieved_gbps": (BYTES_UPDATE + BYTES_NORM) * N / (cev_ms * 1e-3) / 1e9,
             "bytes_per_param": BYTES_UPDATE + BYTES_NORM, "grad_norm": norm, "clip_scale": scale,
+            "norm_ms": norm_ms, "norm_gbps": BYTES_NORM * N / (norm_ms * 1e-3) / 1e9,
             "workload": "same list, g~N(0,5e-3), max_norm=1.0: norm pass + final pass + fused-clip update"}
     clip["frac_of_peak"] = clip["achieved_gbps"] / HBM_PEAK_GBPS
 
+    calibrate = None
     if args.calibrate:
         n_c = 1 << 28
         src = torch.zeros(n_c, dtype=torch.float16, device="cuda:0")
         dst = torch.empty(n_c, dtype=torch.float32, device="cuda:0")
-        for _ in range(3):
-            B.check(B.fp16_to_fp32(dst.data_ptr(), src.data_ptr(), n_c, stream), "rlx_fp16_to_fp32")
-        torch.cuda.synchronize()
+        B.fill_f16(src.data_ptr(), n_c, 77, 0.0, 0.02, stream=stream)
+        conv_ms = time_events(lambda: B.check(B.fp16_to_fp32(dst.data_ptr(), src.data_ptr(), n_c, stream),
+                                              "rlx_fp16_to_fp32"), 2, 5)
+        calibrate = {"kernel": "convert_tile_kernel", "elements": n_c, "bytes": 6 * n_c, "ms": conv_ms,
+                     "gbps": 6 * n_c / (conv_ms * 1e-3) / 1e9}
+        calibrate["frac_of_peak"] = calibrate["gbps"] / HBM_PEAK_GBPS
         del src, dst
 
-    # ---- CPU baseline on a bounded sample of the same workload ----
-    cpu = None
-    if not args.no_cpu:
-        n_s = 32 * 1024 * 1024
-        sample = tuple(grab(k, emb, 0, n_s) for k in ("p", "g", "m", "v"))
-        cpu = cpu_baseline(O, host, sample, hyper, 100)
-
-    # ---- the separate scale pass of the unfused clip (4 bytes per FP16 gradient), last: it shrinks the
-    # gradients on every call; the scale stays the one that the clip leg left on the device ----
+    # ---- the separate scale pass of the unfused clip (4 bytes per FP16 gradient), last on this store: it
+    # shrinks the gradients on every call; the scale stays the one that the clip leg left on the device ----
     scale_ms = time_events(lambda: opt.plan.scale_grads(stream), 1, 5)
     clip["scale_pass_ms"] = scale_ms
     clip["scale_pass_gbps"] = 4 * N / (scale_ms * 1e-3) / 1e9
     clip["unfused_ms_per_step"] = cev_ms + scale_ms
+    chunk_elems, chunks = opt.plan.chunk_elems, opt.plan.num_chunks
+    del opt, st
+    torch.cuda.empty_cache()
 
-    traffic = None
+    # ---- the other configurations, one after the other, each store freed before the next ----
+    configs = {}
+    wanted = [] if args.configs == "none" else list(SECONDARY) if args.configs == "all" else args.configs.split(",")
+    for name in wanted:
+        t0 = time.perf_counter()
+        big = name == "qwen3-8b"
+        configs[name] = measure_workload(name, pkg, host, 10 if big else min(args.steps, 50), 3 if big else min(args.warmup, 10))
+        torch.cuda.empty_cache()
+        log("config %s: update %.4f ms, norm %.4f ms, clip step %.4f ms (%.1f s)" % (
+            name, configs[name]["update_ms"], configs[name]["norm_ms"], configs[name]["clip_step_ms"],
+            time.perf_counter() - t0))
+
+    # ---- CPU baseline on a bounded sample of the same workload ----
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(O, host, sample, g_clip, hyper, 100)
+
+    # HBM bytes per launch of the update kernel as counted by the profiler: recorded beforehand with rocprofv3
+    # (the counters cannot be read from inside this process), only valid for the shipped kernel and chunking
+    traffic, traffic_source = None, None
+    variant = B.get_tuning("update_variant")
     tpath = os.path.join(ROOT, "profiles", "adamw_tile_kernel_qwen3_0.6b_traffic.json")
-    if os.path.exists(tpath):
+    if variant == 0 and args.chunk == 0 and os.path.exists(tpath):
         try:
             traffic = json.load(open(tpath)).get("traffic_bytes_per_launch")
+            traffic_source = "recorded: profiles/adamw_tile_kernel_qwen3_0.6b_traffic.json (rocprofv3 --pmc FETCH_SIZE / " \
+                             "WRITE_SIZE of this command, scaled by a convert stream of known size); not measured in this run"
         except Exception:
             traffic = None
 
     out = {
         "metric": "AdamW params/sec, Qwen3-0.6B step", "value": value, "unit": "params/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "storage": STORAGE,
         "data": "synthetic",
         "config": {"workload": "Qwen3-0.6B tensor list (310 tensors, 596,049,920 params), FP16 p/g, FP32 m/v, "
                                "step 100 after 99 seeded steps, g~N(0,1e-4) with 90% of embedding rows zero, "
                                "no clip; one multi-tensor launch per step",
                    "params": N, "tensors": len(specs), "bytes_per_param": BYTES_UPDATE,
-                   "update_variant": B.get_tuning("update_variant")},
+                   "chunk_elems": chunk_elems, "chunks": chunks, "update_variant": variant},
         "hbm_gbps": BYTES_UPDATE * N * args.steps / wall / 1e9,
         "hbm_frac_of_peak": BYTES_UPDATE * N * args.steps / wall / 1e9 / HBM_PEAK_GBPS,
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic,
-                     "kernel": "adamw_tile_kernel<2,128,1,false,1,0>", "kernel_ms": kernel_ms,
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": traffic, "traffic_source": traffic_source,
+                     "kernel": B.update_variant_name(variant), "kernel_ms": kernel_ms,
                      "algorithmic_bytes_per_launch": BYTES_UPDATE * N,
                      "isolated_launch_ms_min": float(np.min(per)), "isolated_launch_ms_median": float(np.median(per))},
         "cpu_baseline": cpu,
         "clip_step": clip,
+        "configs": configs,
         "parity": "4 sampled slices replayed by the CPU oracle over %d steps: bit-identical" % (100 - first_step),
     }
+    if calibrate:
+        out["calibrate"] = calibrate
     print(json.dumps(out), flush=True)
 
 

@@ -219,16 +219,50 @@ int rlx_plan_adamw(rlx_plan* plan, const rlx_step_params* params, int step_flags
  */
 int rlx_plan_adamw_dev(rlx_plan* plan, const rlx_step_params* dev_params, int step_flags, void* stream);
 
+/*
+ * Steps that need no host at all (a recorded norm + update replayed step after step): the host uploads, once, the
+ * hyper-parameters of the next n_steps steps (learning rates from its scheduler, bias corrections
+ * 1 - powf(beta, t) computed where the reference computes them, include/training/optimizer.h:120-122, so the
+ * values are bit-equal), and every rlx_plan_adamw_scheduled launch reads the current entry from device memory
+ * and then moves on to the next one with a one-lane kernel.  No counterpart in the reference, whose step takes
+ * the values from the host each time (optimizer.h:119-147).
+ *
+ * rlx_plan_schedule_upload: every entry is validated like the arguments of rlx_plan_adamw (finite, bias
+ * corrections not 0: RLX_ERR_BAD_HYPER otherwise, nothing uploaded).  Waits for `stream`, allocates when the
+ * table grows and copies synchronously: call it outside the step loop and outside a graph capture.  The next
+ * scheduled update reads entry 0.
+ * rlx_plan_adamw_scheduled: the update of rlx_plan_adamw_dev with the current entry, then the advance.  After
+ * the last entry has been used, that entry stays current (upload the next window before that happens).
+ * rlx_plan_schedule_position: how many scheduled steps have run since the upload (saturating at n_steps) and
+ * the table's length; waits for `stream`.  Either out pointer may be NULL.
+ */
+int rlx_plan_schedule_upload(rlx_plan* plan, const rlx_step_params* steps, int64_t n_steps, void* stream);
+int rlx_plan_adamw_scheduled(rlx_plan* plan, int step_flags, void* stream);
+int rlx_plan_schedule_position(rlx_plan* plan, int64_t* steps_taken, int64_t* n_steps, void* stream);
+
 /* ------------------------------------------------------------------------------------
  * Launch tuning (process-wide; for measurement).  Unknown keys return RLX_ERR_INVALID_ARG.
  *   "update_variant"  0..N-1   which compiled form of the update kernel: tile shape, XCD swizzle,
  *                              store policy, loads and stores at once or two at a time (0 = default,
- *                              which picks between the last two by what the step writes)
+ *                              which picks between the last two by what the step writes); 10 = 128-bit
+ *                              accesses (8 elements per lane), 11 = that in a persistent grid sized to the
+ *                              CUs striding over the tiles, 12 = that with one workgroup walking a chunk
+ *                              (10-12 with ordinary loads and stores; 13, 14 = 12, 11 with the shipped
+ *                              kernel's non-temporal loads and system-scope non-temporal stores)
  *   "norm_grid"       0 = one workgroup per chunk, >0 = that many persistent workgroups
  *   "norm_nt"         1 = non-temporal loads in the norm pass (default), 0 = plain
+ *   "norm_pack"       512-element chunks per workgroup in the norm pass: 0 = one, 1 = eight (one per
+ *                     wavefront), 2 = thirty-two (four per wavefront, default), 3 = sixteen
+ *   "final_batch"     loads that a lane of the norm's second pass keeps in flight: 8, 16, 32, 40, or
+ *                     0 = chosen from the number of partials (default)
+ *   "convert_variant" rlx_fp16_to_fp32: 0 = 128 lanes x 4 elements per workgroup (default),
+ *                     1 = 128 lanes x 2 elements, 2 = one element per lane, grid-stride,
+ *                     3 = 256 lanes x 4 elements x 2 rounds
  * ---------------------------------------------------------------------------------- */
 int rlx_set_tuning(const char* key, int64_t value);
 int64_t rlx_get_tuning(const char* key);
+/* Name of the kernel instantiation behind an "update_variant" number ("" if out of range). */
+const char* rlx_update_variant_name(int64_t variant);
 
 /* ------------------------------------------------------------------------------------
  * Seeded synthetic inputs, generated on the device (no counterpart in the reference,

@@ -61,6 +61,10 @@ SIGNATURES = {
     "rlx_plan_scale_grads": ([_VP, _VP], _INT),
     "rlx_plan_adamw": ([_VP, C.POINTER(StepParams), _INT, _VP], _INT),
     "rlx_plan_adamw_dev": ([_VP, _VP, _INT, _VP], _INT),
+    "rlx_plan_schedule_upload": ([_VP, C.POINTER(StepParams), _I64, _VP], _INT),
+    "rlx_plan_adamw_scheduled": ([_VP, _INT, _VP], _INT),
+    "rlx_plan_schedule_position": ([_VP, C.POINTER(_I64), C.POINTER(_I64), _VP], _INT),
+    "rlx_update_variant_name": ([_I64], C.c_char_p),
     "rlx_set_tuning": ([C.c_char_p, _I64], _INT),
     "rlx_get_tuning": ([C.c_char_p], _I64),
     "rlx_fill_f16": ([_VP, _I64, _U64, _I64, _F, _F, _U32, _I64, _U32, _VP], _INT),
@@ -70,19 +74,24 @@ SIGNATURES = {
 _lib = None
 
 
+ABI_VERSION = 108        # rlx_version() of the library this binding was written against
+
+
 def load():
-    """Loads the built library, compiling it first if it is missing; raises if that fails (there is no
-    CPU fallback of any kind)."""
+    """Loads the built library.  If it is missing, or was built from other sources than the ones in the tree
+    (the build leaves a hash of its sources next to the library), it is compiled first; if that fails, or the
+    loaded library reports another ABI version than this binding expects, loading raises.  There is no CPU
+    fallback of any kind."""
     global _lib
     if _lib is not None:
         return _lib
-    if not os.path.exists(LIB_PATH):
-        # nothing built yet: compile now (hipcc); if that fails there is nothing to fall back to
-        from . import build as _build
+    from . import build as _build
+    if not _build.is_current():
+        why = "not built" if not os.path.exists(LIB_PATH) else "built from other sources than the tree holds"
         try:
             _build.build_library()
         except Exception as exc:
-            raise RuntimeError("librlx_adamw.so is not built (%s) and building it failed: %s" % (LIB_PATH, exc))
+            raise RuntimeError("librlx_adamw.so is %s (%s) and building it failed: %s" % (why, LIB_PATH, exc))
     try:
         # torch, when present, brings its own HIP runtime: load it first so that this library
         # binds to the same runtime instance as the tensors it is handed.
@@ -94,6 +103,9 @@ def load():
         fn = getattr(lib, name)
         fn.argtypes = args
         fn.restype = res
+    if lib.rlx_version() != ABI_VERSION:
+        raise RuntimeError("librlx_adamw.so reports ABI version %d, this binding expects %d: rebuild the library "
+                           "(python rl.cu_amd/build.py)" % (lib.rlx_version(), ABI_VERSION))
     _lib = lib
     return lib
 
@@ -119,6 +131,12 @@ def set_tuning(key, value):
 
 def get_tuning(key):
     return int(load().rlx_get_tuning(key.encode()))
+
+
+def update_variant_name(variant=None):
+    """Kernel instantiation behind an update_variant number (default: the active one)."""
+    v = get_tuning("update_variant") if variant is None else variant
+    return load().rlx_update_variant_name(v).decode()
 
 
 def adamw_fp16(master_w, model_w, grad, m, v, n, lr, beta1, beta2, eps, weight_decay, bc1, bc2, stream=0):
@@ -219,6 +237,21 @@ class Plan:
 
     def adamw_dev(self, dev_params_ptr, step_flags=CLIP_NONE, stream=0):
         check(load().rlx_plan_adamw_dev(self._h, dev_params_ptr, step_flags, stream), "rlx_plan_adamw_dev")
+
+    def schedule_upload(self, steps, stream=0):
+        """steps: list of StepParams for the coming scheduled steps (validated; blocking)."""
+        arr = (StepParams * len(steps))(*steps)
+        check(load().rlx_plan_schedule_upload(self._h, arr, len(steps), stream), "rlx_plan_schedule_upload")
+
+    def adamw_scheduled(self, step_flags=CLIP_NONE, stream=0):
+        check(load().rlx_plan_adamw_scheduled(self._h, step_flags, stream), "rlx_plan_adamw_scheduled")
+
+    def schedule_position(self, stream=0):
+        """Blocking.  Returns (scheduled steps taken since the upload, length of the table)."""
+        taken, total = _I64(), _I64()
+        check(load().rlx_plan_schedule_position(self._h, C.byref(taken), C.byref(total), stream),
+              "rlx_plan_schedule_position")
+        return taken.value, total.value
 
     def destroy(self):
         if self._h is not None:

@@ -1,4 +1,5 @@
 """Builds librlx_adamw.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree."""
+import hashlib
 import os
 import shutil
 import subprocess
@@ -16,6 +17,28 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wall", "-Wno-unused-command-line-argument",
 ]
+
+
+HEADER = os.path.join(ROOT, "include", "rlx_adamw.h")
+STAMP = OUT + ".srchash"
+
+
+def source_hash():
+    """Hash of everything the library is built from (kernel source, C header, compiler flags)."""
+    h = hashlib.sha256()
+    for path in (SRC, HEADER):
+        with open(path, "rb") as f:
+            h.update(f.read())
+    h.update(" ".join(HIPCC_FLAGS).encode())
+    return h.hexdigest()
+
+
+def is_current():
+    """True if the built library was made from the sources as they are now."""
+    try:
+        return os.path.exists(OUT) and open(STAMP).read().strip() == source_hash()
+    except OSError:
+        return False
 
 
 def hipcc_path():
@@ -36,6 +59,8 @@ def build_library(verbose=False):
     if verbose and err.strip():
         print(err)
     os.replace(OUT + ".tmp", OUT)
+    with open(STAMP, "w") as f:
+        f.write(source_hash() + "\n")
     return OUT
 
 

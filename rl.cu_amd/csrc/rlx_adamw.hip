@@ -60,6 +60,7 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x8 __attribute__((ext_vector_type(8)));
 
 // One chunk of one tensor, pointers already advanced to the chunk's first element.
 struct ChunkRec {
@@ -131,11 +132,14 @@ __device__ __forceinline__ void stg(T* p, T x) {
 
 // Streaming store of the update kernel.  SP = 1 adds the sc1 bit to the non-temporal store
 // (written as inline assembly: the compiler has no spelling for that combination); on MI355X it
-// measured about 1 % faster than the plain non-temporal store for this kernel.
+// measured about 1 % faster than the plain non-temporal store for this kernel.  SP = 0: non-temporal
+// store; SP = 2: ordinary store.
 template <int SP, typename T>
 __device__ __forceinline__ void st_stream(T* p, T x) {
     if constexpr (SP == 0) {
         stg<true>(p, x);
+    } else if constexpr (SP == 2) {
+        stg<false>(p, x);
     } else {
         RLX_GLOBAL T* gp = (RLX_GLOBAL T*)p;
         if constexpr (sizeof(T) == 2) {
@@ -145,9 +149,15 @@ __device__ __forceinline__ void st_stream(T* p, T x) {
             asm volatile("global_store_dword %0, %1, off sc1 nt" ::"v"(gp), "v"(x) : "memory");
         } else if constexpr (sizeof(T) == 8) {
             asm volatile("global_store_dwordx2 %0, %1, off sc1 nt" ::"v"(gp), "v"(x) : "memory");
+        } else if constexpr (sizeof(T) == 16) {
+            // the hardware needs two wait states between a store wider than 64 bits and a write to its data
+            // registers; inside inline assembly the compiler does not insert them itself
+            asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 1" ::"v"(gp), "v"(x) : "memory");
         } else {
-            // a store wider than 8 bytes needs one wait state before its data registers are rewritten
-            asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\ts_nop 0" ::"v"(gp), "v"(x) : "memory");
+            static_assert(sizeof(T) == 32, "store of 2, 4, 8, 16 or 32 bytes");
+            const f32x4 lo = {x[0], x[1], x[2], x[3]}, hi = {x[4], x[5], x[6], x[7]};
+            asm volatile("global_store_dwordx4 %0, %1, off sc1 nt\n\tglobal_store_dwordx4 %0, %2, off offset:16 sc1 nt\n\ts_nop 1"
+                         ::"v"(gp), "v"(lo), "v"(hi) : "memory");
         }
     }
 }
@@ -184,19 +194,28 @@ template <int E> struct Lane;
 template <> struct Lane<1> { typedef uint16_t H; typedef float F; };
 template <> struct Lane<2> { typedef uint32_t H; typedef f32x2 F; };
 template <> struct Lane<4> { typedef u32x2 H; typedef f32x4 F; };
+template <> struct Lane<8> { typedef u32x4 H; typedef f32x8 F; };      // one 128-bit FP16 access, two 128-bit FP32 accesses
 
 template <int E>
 __device__ __forceinline__ void unpack_h(typename Lane<E>::H x, float* out) {
     if constexpr (E == 1) out[0] = h2f(x);
     else if constexpr (E == 2) { out[0] = h2f(x & 0xFFFFu); out[1] = h2f(x >> 16); }
-    else { out[0] = h2f(x[0] & 0xFFFFu); out[1] = h2f(x[0] >> 16); out[2] = h2f(x[1] & 0xFFFFu); out[3] = h2f(x[1] >> 16); }
+    else {
+#pragma unroll
+        for (int k = 0; k < E / 2; k++) { out[2 * k] = h2f(x[k] & 0xFFFFu); out[2 * k + 1] = h2f(x[k] >> 16); }
+    }
 }
 
 template <int E>
 __device__ __forceinline__ typename Lane<E>::H pack_h(const float* w) {
     if constexpr (E == 1) return (uint16_t)f2h(w[0]);
     else if constexpr (E == 2) return f2h(w[0]) | (f2h(w[1]) << 16);
-    else { u32x2 o; o[0] = f2h(w[0]) | (f2h(w[1]) << 16); o[1] = f2h(w[2]) | (f2h(w[3]) << 16); return o; }
+    else {
+        typename Lane<E>::H o;
+#pragma unroll
+        for (int k = 0; k < E / 2; k++) o[k] = f2h(w[2 * k]) | (f2h(w[2 * k + 1]) << 16);
+        return o;
+    }
 }
 
 template <int E>
@@ -248,47 +267,24 @@ __device__ __forceinline__ void update_scalar32(const ChunkRec& r, int64_t i, co
 }
 
 // ---------------------------------------------------------------------------------------
-// Update kernel: one workgroup of BLOCK lanes per tile of E*BLOCK elements.
-// K > 1: workgroups b, b+8, ... land on the same XCD; groups of 8*K tiles are permuted so
-// that each XCD gets K neighbouring tiles.
-// SINGLE: one flat tensor passed by value (the operator API); otherwise the plan's records.
-// SP: 1 = system-scope non-temporal stores, 0 = plain non-temporal stores.
+// Update of one tile: E elements per lane, LANES lanes, TILE = E * LANES elements starting `off` elements into
+// the chunk `r`, of which `left` remain to the end of the chunk / tensor.  `lane` is this lane's index in the tile.
+// SP: 1 = system-scope non-temporal stores, 0 = non-temporal stores, 2 = ordinary stores; NTL: non-temporal loads.
 // PH: 0 = a lane issues the tile's four loads at once; 1 = tiles that write four streams (master copy,
 // gradient clearing) issue their loads, and with a master copy their stores, two at a time.
 // ---------------------------------------------------------------------------------------
 
-template <int E, int BLOCK, int K, bool SINGLE, int SP, int PH>
-__global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
-    const ChunkRec* __restrict__ recs, ChunkRec single, int64_t single_n, int64_t first_tile, int64_t n_tiles,
-    int tiles_per_chunk_log2, Hyper h, const rlx_step_params* __restrict__ dev_params,
-    const NormResult* __restrict__ norm, uint32_t step_flags)
+template <int E, int LANES, int SP, int PH, bool NTL = true>
+__device__ __forceinline__ void update_tile(const ChunkRec& r, int64_t off, int64_t left, int lane, Hyper h,
+                                            const rlx_step_params* __restrict__ dev_params,
+                                            const NormResult* __restrict__ norm, uint32_t step_flags)
 {
-    constexpr int TILE = E * BLOCK;
-    int64_t b = blockIdx.x;
-    if constexpr (K > 1) {
-        const int64_t grp = b / (8 * K), r = b % (8 * K);
-        b = grp * (8 * K) + (r % 8) * K + (r / 8);
-    }
-    const int64_t tile = first_tile + b;
-    if (tile >= n_tiles) return;
-
-    ChunkRec r;
-    int64_t off;         // first element of the tile, relative to r's pointers
-    int64_t left;        // elements from there to the end of the chunk / tensor
-    if constexpr (SINGLE) {
-        r = single;
-        off = tile * TILE;
-        left = single_n - off;
-    } else {
-        r = recs[tile >> tiles_per_chunk_log2];
-        off = (tile & ((1 << tiles_per_chunk_log2) - 1)) * TILE;
-        left = (int64_t)r.count - off;
-    }
+    constexpr int TILE = E * LANES;
     if (left <= 0) return;
     const int n_here = left < TILE ? (int)left : TILE;
     const bool is_f32 = (r.flags & kF32) != 0;
     const int valign = (r.flags >> kValignShift) & 0xF;
-    const int e0 = threadIdx.x * E;
+    const int e0 = lane * E;
     const int64_t i0 = off + e0;
     const bool zero_grads = (step_flags & RLX_STEP_ZERO_GRADS) != 0;
     const bool vec = valign >= E && e0 + E <= n_here;
@@ -339,11 +335,11 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         const bool has_master = r.master != nullptr;
         HV gw;
         FV mw, vw;
-        const auto load_g = [&] { gw = ldg<true>((const HV*)((const uint16_t*)r.g + i0)); };
-        const auto load_mv = [&] { mw = ldg<true>((const FV*)(r.m + i0)); vw = ldg<true>((const FV*)(r.v + i0)); };
+        const auto load_g = [&] { gw = ldg<NTL>((const HV*)((const uint16_t*)r.g + i0)); };
+        const auto load_mv = [&] { mw = ldg<NTL>((const FV*)(r.m + i0)); vw = ldg<NTL>((const FV*)(r.v + i0)); };
         const auto load_w = [&] {
-            if (has_master) unpack_f<E>(ldg<true>((const FV*)(r.master + i0)), w);
-            else unpack_h<E>(ldg<true>((const HV*)((const uint16_t*)r.p + i0)), w);
+            if (has_master) unpack_f<E>(ldg<NTL>((const FV*)(r.master + i0)), w);
+            else unpack_h<E>(ldg<NTL>((const HV*)((const uint16_t*)r.p + i0)), w);
         };
         // A tile that writes four streams (master copy, or gradients cleared) runs faster when a wavefront has
         // two loads in flight at a time instead of four: measured on Qwen3-0.6B with realistic values, 2.69 ->
@@ -377,10 +373,10 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         if (zero_grads) st_stream<SP>((HV*)((uint16_t*)r.g + i0), HV{});
     } else {
         // FP32 parameters (norm weights): the same update, in place (adamw.cu:80-90)
-        unpack_f<E>(ldg<true>((const FV*)((const float*)r.g + i0)), g);
-        unpack_f<E>(ldg<true>((const FV*)(r.m + i0)), m);
-        unpack_f<E>(ldg<true>((const FV*)(r.v + i0)), v);
-        unpack_f<E>(ldg<true>((const FV*)((const float*)r.p + i0)), w);
+        unpack_f<E>(ldg<NTL>((const FV*)((const float*)r.g + i0)), g);
+        unpack_f<E>(ldg<NTL>((const FV*)(r.m + i0)), m);
+        unpack_f<E>(ldg<NTL>((const FV*)(r.v + i0)), v);
+        unpack_f<E>(ldg<NTL>((const FV*)((const float*)r.p + i0)), w);
         if (clip) {
 #pragma unroll
             for (int k = 0; k < E; k++) g[k] = g[k] * scale;
@@ -392,6 +388,79 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         st_stream<SP>((FV*)((float*)r.p + i0), pack_f<E>(w));
         if (zero_grads) st_stream<SP>((FV*)((float*)r.g + i0), FV{});
     }
+}
+
+// ---------------------------------------------------------------------------------------
+// Update kernel, the shipped form: one workgroup of BLOCK lanes per tile of E*BLOCK elements.
+// K > 1: workgroups b, b+8, ... land on the same XCD; groups of 8*K tiles are permuted so
+// that each XCD gets K neighbouring tiles.
+// SINGLE: one flat tensor passed by value (the operator API); otherwise the plan's records.
+// ---------------------------------------------------------------------------------------
+
+template <int E, int BLOCK, int K, bool SINGLE, int SP, int PH, bool NTL>
+__global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
+    const ChunkRec* __restrict__ recs, ChunkRec single, int64_t single_n, int64_t first_tile, int64_t n_tiles,
+    int tiles_per_chunk_log2, Hyper h, const rlx_step_params* __restrict__ dev_params,
+    const NormResult* __restrict__ norm, uint32_t step_flags)
+{
+    constexpr int TILE = E * BLOCK;
+    int64_t b = blockIdx.x;
+    if constexpr (K > 1) {
+        const int64_t grp = b / (8 * K), r = b % (8 * K);
+        b = grp * (8 * K) + (r % 8) * K + (r / 8);
+    }
+    const int64_t tile = first_tile + b;
+    if (tile >= n_tiles) return;
+
+    ChunkRec r;
+    int64_t off;         // first element of the tile, relative to r's pointers
+    int64_t left;        // elements from there to the end of the chunk / tensor
+    if constexpr (SINGLE) {
+        r = single;
+        off = tile * TILE;
+        left = single_n - off;
+    } else {
+        r = recs[tile >> tiles_per_chunk_log2];
+        off = (tile & ((1 << tiles_per_chunk_log2) - 1)) * TILE;
+        left = (int64_t)r.count - off;
+    }
+    update_tile<E, BLOCK, SP, PH, NTL>(r, off, left, threadIdx.x, h, dev_params, norm, step_flags);
+}
+
+// ---------------------------------------------------------------------------------------
+// Two other shapes of the same update, kept compiled so that the choice of the shipped one can be measured
+// again at any time (tuning key "update_variant"); they give the same bits.
+//
+// adamw_persistent_kernel: a grid sized to the device (a fixed number of workgroups per CU) whose wavefronts
+// stride over the tiles, 8 elements per lane: one 128-bit access per FP16 stream and two per FP32 stream.
+// adamw_chunk_kernel: one workgroup per chunk that walks its chunk in groups of E*BLOCK elements.
+// ---------------------------------------------------------------------------------------
+
+template <int E, int WAVES, int SP, bool NTL>
+__global__ __launch_bounds__(64 * WAVES) void adamw_persistent_kernel(
+    const ChunkRec* __restrict__ recs, int64_t n_tiles, int tiles_per_chunk_log2, Hyper h,
+    const rlx_step_params* __restrict__ dev_params, const NormResult* __restrict__ norm, uint32_t step_flags)
+{
+    constexpr int TILE = E * 64;                                  // one wavefront per tile
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;   // wave: uniform, so records come by scalar loads
+    for (int64_t tile = (int64_t)blockIdx.x * WAVES + wave; tile < n_tiles; tile += (int64_t)gridDim.x * WAVES) {
+        const ChunkRec r = recs[tile >> tiles_per_chunk_log2];
+        const int64_t off = (tile & ((1 << tiles_per_chunk_log2) - 1)) * TILE;
+        update_tile<E, 64, SP, 0, NTL>(r, off, (int64_t)r.count - off, lane, h, dev_params, norm, step_flags);
+    }
+}
+
+template <int E, int BLOCK, int SP, bool NTL>
+__global__ __launch_bounds__(BLOCK) void adamw_chunk_kernel(
+    const ChunkRec* __restrict__ recs, int64_t first_chunk, int64_t n_chunks, Hyper h,
+    const rlx_step_params* __restrict__ dev_params, const NormResult* __restrict__ norm, uint32_t step_flags)
+{
+    constexpr int TILE = E * BLOCK;
+    const int64_t c = first_chunk + blockIdx.x;
+    if (c >= n_chunks) return;
+    const ChunkRec r = recs[c];
+    for (int64_t off = 0; off < (int64_t)r.count; off += TILE)
+        update_tile<E, BLOCK, SP, 0, NTL>(r, off, (int64_t)r.count - off, threadIdx.x, h, dev_params, norm, step_flags);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -423,15 +492,23 @@ __device__ __forceinline__ ChunkRec pool_chunk(const PoolPair& pp, int64_t c) {
 }
 
 // POOLS: the chunks come from `pools` (two flat buffers passed by value) instead of the table `recs`.
-template <bool NT, int BLOCK, bool POOLS = false>
-__global__ __launch_bounds__(BLOCK) void sumsq_partials_kernel(
+// PACK > 1 (only with BLOCK = 64, i.e. 512-element chunks): the workgroup has PACK wavefronts and each takes
+// a chunk of its own, PACK consecutive chunks per workgroup.  A list of thousands of small tensors has tens of
+// thousands of such chunks, and one single-wavefront workgroup per chunk is bound by the rate at which
+// workgroups are dispatched; the sum inside a chunk and its slot are the same either way.
+template <bool NT, int BLOCK, bool POOLS = false, int PACK = 1>
+__global__ __launch_bounds__(BLOCK * PACK) void sumsq_partials_kernel(
     const ChunkRec* __restrict__ recs, PoolPair pools, int64_t n_chunks, double* __restrict__ partials)
 {
+    static_assert(PACK == 1 || BLOCK == 64, "several chunks per workgroup only with one wavefront per chunk");
     constexpr int kNormGroup = BLOCK * kVec;
     __shared__ float wave_sum[BLOCK / 64];
-    const int tid = threadIdx.x;
+    // which of the workgroup's PACK chunks: the wavefront's number, made known to the compiler as uniform
+    // across the wavefront so that the chunk's record is still fetched with scalar loads
+    const int tid = PACK == 1 ? (int)threadIdx.x : (int)(threadIdx.x & 63);
+    const int sub = PACK == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 
-    for (int64_t c = blockIdx.x; c < n_chunks; c += gridDim.x) {
+    for (int64_t c = (int64_t)blockIdx.x * PACK + sub; c < n_chunks; c += (int64_t)gridDim.x * PACK) {
         ChunkRec r;
         if constexpr (POOLS) r = pool_chunk(pools, c);
         else r = recs[c];
@@ -471,6 +548,20 @@ __global__ __launch_bounds__(BLOCK) void sumsq_partials_kernel(
                         acc = acc + a * a;
                         acc = acc + b * b;
                     }
+                } else if (aligned && off < count) {
+                    // the tensor's last, partial group: its 16-byte granule starts inside the tensor, so one
+                    // aligned load cannot leave the tensor's last page; what lies beyond the end is read but
+                    // counts as zero (acc + 0 leaves a sum of squares as it is).  Element by element this
+                    // lane would wait for up to seven loads one after another, and its workgroup with it.
+                    u32x4 x = ldg<NT>((const u32x4*)(g + off));
+                    const int valid = (int)(count - off);
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        float a = 2 * k < valid ? h2f(x[k] & 0xFFFFu) : 0.0f;
+                        float b = 2 * k + 1 < valid ? h2f(x[k] >> 16) : 0.0f;
+                        acc = acc + a * a;
+                        acc = acc + b * b;
+                    }
                 } else {
                     for (int64_t i = off; i < off + kVec && i < count; i++) {
                         float a = h2f(ldg<NT>(g + i));
@@ -488,6 +579,15 @@ __global__ __launch_bounds__(BLOCK) void sumsq_partials_kernel(
                     for (int k = 0; k < 4; k++) acc = acc + x0[k] * x0[k];
 #pragma unroll
                     for (int k = 0; k < 4; k++) acc = acc + x1[k] * x1[k];
+                } else if (aligned && off < count) {
+                    // partial last group, as above; the second 16-byte granule is only read if it starts inside
+                    const int valid = (int)(count - off);
+                    f32x4 x0 = ldg<NT>((const f32x4*)(g + off)), x1 = {0.0f, 0.0f, 0.0f, 0.0f};
+                    if (valid > 4) x1 = ldg<NT>((const f32x4*)(g + off) + 1);
+#pragma unroll
+                    for (int k = 0; k < 4; k++) { const float a = k < valid ? x0[k] : 0.0f; acc = acc + a * a; }
+#pragma unroll
+                    for (int k = 0; k < 4; k++) { const float a = 4 + k < valid ? x1[k] : 0.0f; acc = acc + a * a; }
                 } else {
                     for (int64_t i = off; i < off + kVec && i < count; i++) {
                         float a = ldg<NT>(g + i);
@@ -499,21 +599,111 @@ __global__ __launch_bounds__(BLOCK) void sumsq_partials_kernel(
 
 #pragma unroll
         for (int mask = 32; mask >= 1; mask >>= 1) acc = acc + __shfl_xor(acc, mask, 64);
-        if ((tid & 63) == 0) wave_sum[tid >> 6] = acc;
-        __syncthreads();
-        if (tid == 0) {
-            double total = 0.0;
+        if constexpr (BLOCK == 64) {
+            // one wavefront per chunk: its sum is the chunk's partial (0.0 + x in FP64, as below, is x)
+            if (tid == 0) partials[c] = (double)acc;
+        } else {
+            if ((tid & 63) == 0) wave_sum[tid >> 6] = acc;
+            __syncthreads();
+            if (tid == 0) {
+                double total = 0.0;
 #pragma unroll
-            for (int w = 0; w < BLOCK / 64; w++) total += (double)wave_sum[w];
-            partials[c] = total;
+                for (int w = 0; w < BLOCK / 64; w++) total += (double)wave_sum[w];
+                partials[c] = total;
+            }
+            __syncthreads();
         }
-        __syncthreads();
+    }
+}
+
+// Norm pass 1 for 512-element chunks (lists of thousands of small tensors): a chunk is at most one 8-element
+// group per lane of one wavefront, so a wavefront takes CPW consecutive chunks at once (records and data of all
+// of them requested before the first is used) and a workgroup of WAVES wavefronts WAVES * CPW chunks.  With one
+// chunk per wavefront the pass is bound by latency: record, data, butterfly, one after another, for each of
+// tens of thousands of chunks.  The sum inside a chunk and its slot are those of the general kernel above with
+// BLOCK = 64 (lane t adds its group's elements in order, xor butterfly), so the results are the same bits.
+template <bool NT, bool POOLS, int WAVES, int CPW>
+__global__ __launch_bounds__(64 * WAVES) void sumsq_small_chunks_kernel(
+    const ChunkRec* __restrict__ recs, PoolPair pools, int64_t n_chunks, double* __restrict__ partials)
+{
+    const int lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));    // uniform: records by scalar loads
+    const int64_t first = ((int64_t)blockIdx.x * WAVES + wave) * CPW;
+    if (first >= n_chunks) return;
+
+    const char* g[CPW];
+    int valid[CPW];          // elements of chunk j that belong to this lane's group (0..8)
+    bool f32[CPW], fast[CPW];
+    u32x4 a[CPW], b[CPW];
+#pragma unroll
+    for (int j = 0; j < CPW; j++) {
+        ChunkRec r;
+        r.g = nullptr; r.count = 0; r.flags = 0;
+        if (first + j < n_chunks) {
+            if constexpr (POOLS) r = pool_chunk(pools, first + j);
+            else r = recs[first + j];
+        }
+        g[j] = (const char*)r.g;
+        f32[j] = (r.flags & kF32) != 0;
+        fast[j] = ((r.flags >> kValignShift) & 0xF) >= 8;
+        int left = (r.flags & RLX_TENSOR_FROZEN) ? 0 : (int)r.count - lane * kVec;   // a frozen tensor counts as zero
+        valid[j] = left < 0 ? 0 : left > kVec ? kVec : left;
+    }
+#pragma unroll
+    for (int j = 0; j < CPW; j++) {
+        a[j] = u32x4{0u, 0u, 0u, 0u};
+        b[j] = u32x4{0u, 0u, 0u, 0u};
+        // aligned chunks: whole 16-byte granules that start inside the tensor (what lies beyond its end is
+        // read but not used, see the general kernel)
+        if (fast[j] && valid[j] > 0) {
+            const u32x4* src = (const u32x4*)(g[j] + (size_t)lane * (f32[j] ? 32 : 16));
+            a[j] = ldg<NT>(src);
+            if (f32[j] && valid[j] > 4) b[j] = ldg<NT>(src + 1);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < CPW; j++) {
+        float acc = 0.0f;
+        if (fast[j]) {
+            if (!f32[j]) {
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const float x = 2 * k < valid[j] ? h2f(a[j][k] & 0xFFFFu) : 0.0f;
+                    const float y = 2 * k + 1 < valid[j] ? h2f(a[j][k] >> 16) : 0.0f;
+                    acc = acc + x * x;
+                    acc = acc + y * y;
+                }
+            } else {
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const uint32_t w = a[j][k];      // (a bit cast applied directly to a vector element took element 0 every time)
+                    const float x = k < valid[j] ? __builtin_bit_cast(float, w) : 0.0f;
+                    acc = acc + x * x;
+                }
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    const uint32_t w = b[j][k];
+                    const float x = 4 + k < valid[j] ? __builtin_bit_cast(float, w) : 0.0f;
+                    acc = acc + x * x;
+                }
+            }
+        } else {
+            for (int e = 0; e < valid[j]; e++) {          // a chunk that is not 16-byte aligned: element by element
+                const float x = f32[j] ? ldg<NT>((const float*)g[j] + lane * kVec + e)
+                                       : h2f(ldg<NT>((const uint16_t*)g[j] + lane * kVec + e));
+                acc = acc + x * x;
+            }
+        }
+#pragma unroll
+        for (int mask = 32; mask >= 1; mask >>= 1) acc = acc + __shfl_xor(acc, mask, 64);
+        if (lane == 0 && first + j < n_chunks) partials[first + j] = (double)acc;
     }
 }
 
 // Norm pass 2: one workgroup, fixed order.  Thread t adds partials t, t+1024, ... in FP64,
 // then a halving tree through LDS.  Writes the sum, the norm and the clip scale
 // (trainer.h:341-345: strict '>' and +1e-6f in the denominator).
+template <int BATCH>
 __global__ __launch_bounds__(kFinalBlock) void sumsq_final_kernel(
     const double* __restrict__ partials, int64_t n_partials, float max_norm, NormResult* __restrict__ out)
 {
@@ -521,18 +711,18 @@ __global__ __launch_bounds__(kFinalBlock) void sumsq_final_kernel(
     const int tid = threadIdx.x;
     double a = 0.0;
     int64_t i = tid;
-    // sixteen independent loads in flight, added in index order: the same sum as one at a time.  Slots beyond
+    // BATCH independent loads in flight, added in index order: the same sum as one at a time.  Slots beyond
     // the end read as +0.0, which leaves a sum of squares (never negative zero) unchanged bit for bit; without
     // them the last few partials of every lane would each cost a round trip of their own.
-    for (; i < n_partials; i += 16 * (int64_t)kFinalBlock) {
-        double x[16];
+    for (; i < n_partials; i += BATCH * (int64_t)kFinalBlock) {
+        double x[BATCH];
 #pragma unroll
-        for (int k = 0; k < 16; k++) {
+        for (int k = 0; k < BATCH; k++) {
             const int64_t j = i + k * (int64_t)kFinalBlock;
             x[k] = j < n_partials ? partials[j] : 0.0;
         }
 #pragma unroll
-        for (int k = 0; k < 16; k++) a += x[k];
+        for (int k = 0; k < BATCH; k++) a += x[k];
     }
     acc[tid] = a;
     __syncthreads();
@@ -612,11 +802,58 @@ __global__ __launch_bounds__(256) void scale_f32_kernel(float* __restrict__ x, f
     }
 }
 
+// dst[i] = (float)src[i] as a stream (the FP32 master copy made from the FP16 weights, optimizer.h:46-57,242).
+// One workgroup of LANES lanes per LANES*E*ROUNDS elements (shipped: 128 lanes x 4 elements, one round: a
+// 64-bit load and a 128-bit store per lane); per lane and round one access of E halves and one of E floats, every instruction contiguous across the wavefront, all loads issued before the first use,
+// non-temporal loads and system-scope non-temporal stores.  Workgroups whose span is not whole or not aligned
+// go element by element.
+template <int LANES, int E, int ROUNDS>
+__global__ __launch_bounds__(LANES) void convert_tile_kernel(float* __restrict__ dst, const uint16_t* __restrict__ src,
+                                                             int64_t n, int vec_ok)
+{
+    constexpr int PER = LANES * E;
+    typedef typename Lane<E>::H HV;
+    typedef typename Lane<E>::F FV;
+    const int64_t base = (int64_t)blockIdx.x * (PER * ROUNDS) + (int64_t)threadIdx.x * E;
+    if (vec_ok && (int64_t)(blockIdx.x + 1) * (PER * ROUNDS) <= n) {
+        HV x[ROUNDS];
+#pragma unroll
+        for (int r = 0; r < ROUNDS; r++) x[r] = ldg<true>((const HV*)(src + base + r * PER));
+#pragma unroll
+        for (int r = 0; r < ROUNDS; r++) {
+            float f[E];
+            unpack_h<E>(x[r], f);
+            st_stream<1>((FV*)(dst + base + r * PER), pack_f<E>(f));
+        }
+    } else {
+        for (int r = 0; r < ROUNDS; r++)
+            for (int e = 0; e < E; e++) {
+                const int64_t i = base + r * PER + e;
+                if (i < n) dst[i] = h2f(src[i]);
+            }
+    }
+}
+
+// The plain form: one element per lane, grid-stride (kept for comparison: tuning key "convert_variant" = 2).
 __global__ __launch_bounds__(256) void fp16_to_fp32_kernel(float* __restrict__ dst,
                                                            const uint16_t* __restrict__ src, int64_t n)
 {
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256)
         dst[i] = h2f(src[i]);
+}
+
+// After an update that read the current entry of a plan's step table: move on to the next entry, so that the
+// next (replayed) update reads new hyper-parameters without the host.  Beyond the end of the table the last
+// entry stays current; *taken counts the scheduled steps so far, saturating at n.
+__global__ __launch_bounds__(64) void schedule_advance_kernel(const rlx_step_params* __restrict__ table, int64_t n,
+                                                              int64_t* __restrict__ taken,
+                                                              rlx_step_params* __restrict__ current)
+{
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    int64_t next = *taken + 1;
+    if (next < n) *current = table[next];
+    if (next > n) next = n;
+    *taken = next;
 }
 
 // Zero fill as a kernel (a memset node recorded into a HIP graph is not reliable on every
@@ -705,9 +942,14 @@ struct Tuning {
     int64_t update_variant = 0;
     int64_t norm_grid = 0;
     int64_t norm_nt = 1;
+    int64_t norm_pack = 2;          // 512-element chunks per workgroup: 0 = one, 1 = eight (a wavefront each),
+                                    // 2 = thirty-two (four per wavefront, the default), 3 = sixteen
+    int64_t convert_variant = 0;
+    int64_t final_batch = 0;        // loads in flight per lane in the second pass of the norm; 0 = by the number of partials
 } g_tuning;
 
-constexpr int kNumUpdateVariants = 10;
+constexpr int kNumUpdateVariants = 15;
+constexpr int kNumConvertVariants = 4;
 constexpr int64_t kMaxTilesPerLaunch = 1 << 23;   // workgroups per launch; times 256 lanes stays below 2^32
 constexpr int64_t kMaxNormGrid = 1 << 22;
 
@@ -780,26 +1022,95 @@ ChunkRec make_rec(const rlx_tensor_desc& d, int64_t start, int64_t count) {
     return r;
 }
 
-template <int E, int BLOCK, int K, bool SINGLE, int SP, int PH = 0>
-void launch_variant(const ChunkRec* recs, const ChunkRec& single, int64_t single_n, int64_t n_elems_or_tiles,
-                    int chunk_log2, const Hyper& h, const rlx_step_params* dev_params, const NormResult* norm,
-                    uint32_t step_flags, hipStream_t s) {
+// Every launch is checked where it is made, so that a failure names the launch: returns hipSuccess or the
+// first error.
+template <int E, int BLOCK, int K, bool SINGLE, int SP, int PH = 0, bool NTL = true>
+hipError_t launch_variant(const ChunkRec* recs, const ChunkRec& single, int64_t single_n, int64_t n_elems_or_chunks,
+                          int chunk_log2, const Hyper& h, const rlx_step_params* dev_params, const NormResult* norm,
+                          uint32_t step_flags, hipStream_t s) {
     constexpr int TILE = E * BLOCK;
     int64_t n_tiles;
     int tpc_log2 = 0;
     if constexpr (SINGLE) {
-        n_tiles = (n_elems_or_tiles + TILE - 1) / TILE;
+        n_tiles = (n_elems_or_chunks + TILE - 1) / TILE;
     } else {
         tpc_log2 = chunk_log2 - __builtin_ctz(TILE);
-        n_tiles = n_elems_or_tiles << tpc_log2;          // n_chunks * tiles per chunk
+        n_tiles = n_elems_or_chunks << tpc_log2;          // n_chunks * tiles per chunk
     }
     for (int64_t first = 0; first < n_tiles; first += kMaxTilesPerLaunch) {
         int64_t here = n_tiles - first < kMaxTilesPerLaunch ? n_tiles - first : kMaxTilesPerLaunch;
         here = (here + 8 * K - 1) / (8 * K) * (8 * K);   // whole swizzle groups; the excess exits at once
-        adamw_tile_kernel<E, BLOCK, K, SINGLE, SP, PH><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(
+        adamw_tile_kernel<E, BLOCK, K, SINGLE, SP, PH, NTL><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(
             recs, single, single_n, first, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
     }
+    return hipSuccess;
 }
+
+// Workgroups per CU of the persistent form: four wavefronts each, eight fill a CU's wavefront slots.
+constexpr int kPersistentWaves = 4, kPersistentPerCU = 8;
+
+int compute_units() {
+    static int cached[kMaxDevices];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) return 256;
+    if (!cached[dev]) {
+        int cu = 0;
+        if (hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0) cu = 256;
+        cached[dev] = cu;
+    }
+    return cached[dev];
+}
+
+template <int SP, bool NTL>
+hipError_t launch_persistent(const ChunkRec* recs, int64_t n_chunks, int chunk_log2, const Hyper& h,
+                             const rlx_step_params* dev_params, const NormResult* norm, uint32_t step_flags,
+                             hipStream_t s) {
+    constexpr int E = 8, TILE = E * 64;
+    const int tpc_log2 = chunk_log2 - __builtin_ctz(TILE);
+    const int64_t n_tiles = n_chunks << tpc_log2;
+    int64_t grid = (int64_t)compute_units() * kPersistentPerCU;
+    const int64_t need = (n_tiles + kPersistentWaves - 1) / kPersistentWaves;
+    if (grid > need) grid = need;
+    adamw_persistent_kernel<E, kPersistentWaves, SP, NTL><<<dim3((unsigned)grid), dim3(64 * kPersistentWaves), 0, s>>>(
+        recs, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
+    return hipGetLastError();
+}
+
+template <int SP, bool NTL>
+hipError_t launch_per_chunk(const ChunkRec* recs, int64_t n_chunks, const Hyper& h, const rlx_step_params* dev_params,
+                            const NormResult* norm, uint32_t step_flags, hipStream_t s) {
+    for (int64_t first = 0; first < n_chunks; first += kMaxTilesPerLaunch) {
+        const int64_t here = n_chunks - first < kMaxTilesPerLaunch ? n_chunks - first : kMaxTilesPerLaunch;
+        adamw_chunk_kernel<8, 256, SP, NTL><<<dim3((unsigned)here), dim3(256), 0, s>>>(recs, first, n_chunks, h, dev_params, norm,
+                                                                               step_flags);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+// The compiled forms of the update ("update_variant"), by number; 0 is what ships.
+const char* const kVariantNames[kNumUpdateVariants] = {
+    "adamw_tile_kernel<2,128,1,*,1,0|1>",      // 0: 2 elements x 128 lanes, sc1 nt stores; loads at once, or two
+                                               //    at a time when the step writes four streams
+    "adamw_tile_kernel<2,128,2,*,1,0>",        // 1: with the XCD swizzle
+    "adamw_tile_kernel<2,64,1,*,1,0>",         // 2
+    "adamw_tile_kernel<4,64,1,*,1,0>",         // 3
+    "adamw_tile_kernel<2,256,1,*,1,0>",        // 4
+    "adamw_tile_kernel<1,256,1,*,1,0>",        // 5
+    "adamw_tile_kernel<4,128,1,*,1,0>",        // 6
+    "adamw_tile_kernel<2,128,1,*,0,0>",        // 7: plain nt stores
+    "adamw_tile_kernel<2,128,1,*,1,0>",        // 8: always loads at once
+    "adamw_tile_kernel<2,128,1,*,1,1>",        // 9: always the two-at-a-time form
+    "adamw_tile_kernel<8,64,1,*,2,0,false>",   // 10: 128-bit FP16 / 2 x 128-bit FP32 accesses per lane, one wavefront per
+                                               //     512-element tile, ordinary loads and stores
+    "adamw_persistent_kernel<8,4,2,false>",    // 11: 128-bit accesses, grid sized to the CUs, wavefronts stride over the tiles
+    "adamw_chunk_kernel<8,256,2,false>",       // 12: 128-bit accesses, one 256-lane workgroup walks a whole chunk
+    "adamw_chunk_kernel<8,256,1,true>",        // 13: the same with the shipped kernel's non-temporal loads and sc1 nt stores
+    "adamw_persistent_kernel<8,4,1,true>",     // 14: the persistent form with those
+};
 
 // any_master: some tensor of the launch has an FP32 master copy.  Such launches, and those that clear the
 // gradients, write four streams per tile and take the form of the kernel that splits its loads and stores.
@@ -808,23 +1119,33 @@ int launch_update(const ChunkRec* recs, const ChunkRec& single, int64_t single_n
                   const Hyper& h, const rlx_step_params* dev_params, const NormResult* norm, uint32_t step_flags,
                   bool any_master, hipStream_t s) {
     const bool four_streams = any_master || (step_flags & RLX_STEP_ZERO_GRADS) != 0;
-    switch (g_tuning.update_variant) {
+    hipError_t e = hipSuccess;
+#define RLX_V(...) e = launch_variant<__VA_ARGS__>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s)
+    int64_t variant = g_tuning.update_variant;
+    if (SINGLE && variant >= 11) variant = 0;      // the table-walking forms have no flat-tensor counterpart
+    switch (variant) {
     default:
     case 0:
-        if (four_streams) launch_variant<2, 128, 1, SINGLE, 1, 1>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s);
-        else launch_variant<2, 128, 1, SINGLE, 1, 0>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s);
+        if (four_streams) RLX_V(2, 128, 1, SINGLE, 1, 1);
+        else RLX_V(2, 128, 1, SINGLE, 1, 0);
         break;
-    case 1: launch_variant<2, 128, 2, SINGLE, 1>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
-    case 2: launch_variant<2, 64, 1, SINGLE, 1>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
-    case 3: launch_variant<4, 64, 1, SINGLE, 1>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
-    case 4: launch_variant<2, 256, 1, SINGLE, 1>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
-    case 5: launch_variant<1, 256, 1, SINGLE, 1>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
-    case 6: launch_variant<4, 128, 1, SINGLE, 1>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
-    case 7: launch_variant<2, 128, 1, SINGLE, 0>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
-    case 8: launch_variant<2, 128, 1, SINGLE, 1, 0>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
-    case 9: launch_variant<2, 128, 1, SINGLE, 1, 1>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 1: RLX_V(2, 128, 2, SINGLE, 1); break;
+    case 2: RLX_V(2, 64, 1, SINGLE, 1); break;
+    case 3: RLX_V(4, 64, 1, SINGLE, 1); break;
+    case 4: RLX_V(2, 256, 1, SINGLE, 1); break;
+    case 5: RLX_V(1, 256, 1, SINGLE, 1); break;
+    case 6: RLX_V(4, 128, 1, SINGLE, 1); break;
+    case 7: RLX_V(2, 128, 1, SINGLE, 0); break;
+    case 8: RLX_V(2, 128, 1, SINGLE, 1, 0); break;
+    case 9: RLX_V(2, 128, 1, SINGLE, 1, 1); break;
+    case 10: RLX_V(8, 64, 1, SINGLE, 2, 0, false); break;
+    case 11: if constexpr (!SINGLE) e = launch_persistent<2, false>(recs, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 12: if constexpr (!SINGLE) e = launch_per_chunk<2, false>(recs, n, h, dev_params, norm, step_flags, s); break;
+    case 13: if constexpr (!SINGLE) e = launch_per_chunk<1, true>(recs, n, h, dev_params, norm, step_flags, s); break;
+    case 14: if constexpr (!SINGLE) e = launch_persistent<1, true>(recs, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
     }
-    RLX_HIP(hipGetLastError());
+#undef RLX_V
+    if (e != hipSuccess) return hip_fail(e, "update kernel launch");
     return RLX_OK;
 }
 
@@ -845,7 +1166,8 @@ int flat_update(void* p, const void* g, float* m, float* v, float* master, int64
 }
 
 // Zero fill of [dst, dst + nbytes): 128-bit stores over the 16-byte-aligned body, bytes at the edges.
-void clear_range(void* dst, int64_t nbytes, hipStream_t s) {
+// Returns the first launch error, if any.
+hipError_t clear_range(void* dst, int64_t nbytes, hipStream_t s) {
     uint8_t* b = (uint8_t*)dst;
     int64_t n_head = (int64_t)((16 - ((uintptr_t)b & 15)) & 15);
     if (n_head > nbytes) n_head = nbytes;
@@ -856,9 +1178,12 @@ void clear_range(void* dst, int64_t nbytes, hipStream_t s) {
     for (int64_t first = 0; first < n_vec; first += per_launch) {
         const int64_t here = n_vec - first < per_launch ? n_vec - first : per_launch;
         clear_body_kernel<<<dim3((unsigned)((here + 255) / 256)), dim3(256), 0, s>>>(body + first, here);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
     }
     if (n_head || n_tail)
         clear_edges_kernel<<<dim3(1), dim3(64), 0, s>>>(b, (int)n_head, b + n_head + n_vec * 16, (int)n_tail);
+    return hipGetLastError();
 }
 
 }  // namespace
@@ -879,6 +1204,12 @@ struct rlx_plan {
     double* d_partials;
     NormResult* d_norm;
     NormResult* h_norm;      // pinned
+    // host-free replay: a table of per-step hyper-parameters on the device, the entry that the next scheduled
+    // update reads (d_current) and the count of scheduled steps taken (d_taken); all null until a table is uploaded
+    rlx_step_params* d_sched;
+    int64_t sched_cap, sched_len;
+    rlx_step_params* d_current;
+    int64_t* d_taken;
 };
 
 namespace {
@@ -908,6 +1239,19 @@ void launch_scale_groups(const rlx_plan* p, hipStream_t s) {
     }
 }
 
+// Pass 2.  How many loads a lane keeps in flight only changes the speed, not the order of the sum.
+void launch_final(const double* partials, int64_t n, float max_norm, NormResult* result, hipStream_t s) {
+    int64_t batch = g_tuning.final_batch;
+    if (batch == 0) {          // automatic: about as many as a lane has partials to add, so that few slots are empty
+        const int64_t per_lane = (n + kFinalBlock - 1) / kFinalBlock;
+        batch = per_lane <= 8 ? 8 : per_lane <= 16 ? 16 : per_lane <= 32 ? 32 : 40;
+    }
+    if (batch == 8) sumsq_final_kernel<8><<<dim3(1), dim3(kFinalBlock), 0, s>>>(partials, n, max_norm, result);
+    else if (batch == 32) sumsq_final_kernel<32><<<dim3(1), dim3(kFinalBlock), 0, s>>>(partials, n, max_norm, result);
+    else if (batch == 40) sumsq_final_kernel<40><<<dim3(1), dim3(kFinalBlock), 0, s>>>(partials, n, max_norm, result);
+    else sumsq_final_kernel<16><<<dim3(1), dim3(kFinalBlock), 0, s>>>(partials, n, max_norm, result);
+}
+
 // Both passes of the norm over n_chunks chunks (from the table `recs`, or from `pools` if POOLS): one FP64
 // partial per chunk into `partials`, then the fixed-order sum and the clip rule into `result`.
 template <bool POOLS>
@@ -928,10 +1272,33 @@ int launch_norm(const ChunkRec* recs, const PoolPair& pools, int64_t n_chunks, i
     if (lanes >= 512) RLX_NORM_LAUNCH(512);
     else if (lanes == 256) RLX_NORM_LAUNCH(256);
     else if (lanes == 128) RLX_NORM_LAUNCH(128);
-    else RLX_NORM_LAUNCH(64);
+    else if (g_tuning.norm_pack == 0) RLX_NORM_LAUNCH(64);
+    else if (g_tuning.norm_pack == 1) {
+        // 512-element chunks: eight wavefronts per workgroup, one chunk each
+        constexpr int PACK = 8;
+        const dim3 pgrid((unsigned)((g + PACK - 1) / PACK));
+        if (g_tuning.norm_nt)
+            sumsq_partials_kernel<true, 64, POOLS, PACK><<<pgrid, dim3(64 * PACK), 0, s>>>(recs, pools, n_chunks, partials);
+        else
+            sumsq_partials_kernel<false, 64, POOLS, PACK><<<pgrid, dim3(64 * PACK), 0, s>>>(recs, pools, n_chunks, partials);
+    } else {
+        // 512-element chunks, the default: eight wavefronts per workgroup, four (or two) chunks each
+#define RLX_SMALL(W, C)                                                                                          \
+    do {                                                                                                         \
+        const int64_t per_wg = (W) * (C);                                                                        \
+        const dim3 pgrid((unsigned)((n_chunks + per_wg - 1) / per_wg));                                          \
+        if (g_tuning.norm_nt)                                                                                    \
+            sumsq_small_chunks_kernel<true, POOLS, W, C><<<pgrid, dim3(64 * (W)), 0, s>>>(recs, pools, n_chunks, partials);  \
+        else                                                                                                     \
+            sumsq_small_chunks_kernel<false, POOLS, W, C><<<pgrid, dim3(64 * (W)), 0, s>>>(recs, pools, n_chunks, partials); \
+    } while (0)
+        if (g_tuning.norm_pack == 3) RLX_SMALL(8, 2);
+        else RLX_SMALL(8, 4);
+#undef RLX_SMALL
+    }
 #undef RLX_NORM_LAUNCH
     RLX_HIP(hipGetLastError());
-    sumsq_final_kernel<<<dim3(1), dim3(kFinalBlock), 0, s>>>(partials, n_chunks, max_norm, result);
+    launch_final(partials, n_chunks, max_norm, result, s);
     RLX_HIP(hipGetLastError());
     return RLX_OK;
 }
@@ -953,8 +1320,7 @@ int plan_update(const rlx_plan* p, const Hyper& h, const rlx_step_params* dev_pa
         if (st != RLX_OK) return st;
     }
     if (clear) {
-        for (const auto& r : p->idle_grads) clear_range(r.first, r.second, s);
-        RLX_HIP(hipGetLastError());
+        for (const auto& r : p->idle_grads) RLX_HIP(clear_range(r.first, r.second, s));
     }
     return RLX_OK;
 }
@@ -980,7 +1346,7 @@ const char* rlx_status_string(int status) {
 
 const char* rlx_last_hip_error(void) { return g_hip_error; }
 
-int rlx_version(void) { return 107; }
+int rlx_version(void) { return 108; }
 
 int rlx_adamw_fp16(float* master_w, uint16_t* model_w, const uint16_t* grad, float* m, float* v, int64_t n,
                    float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -1000,10 +1366,32 @@ int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream) {
     if (n <= 0) return RLX_OK;
     if (!dst || !src) return RLX_ERR_INVALID_ARG;
     if (!is_aligned(dst, 4) || !is_aligned(src, 2)) return RLX_ERR_MISALIGNED;
-    int64_t grid = (n + 255) / 256;
-    if (grid > 65536) grid = 65536;
-    fp16_to_fp32_kernel<<<dim3((unsigned)grid), dim3(256), 0, (hipStream_t)stream>>>(dst, src, n);
-    RLX_HIP(hipGetLastError());
+    hipStream_t s = (hipStream_t)stream;
+    if (g_tuning.convert_variant == 2) {
+        int64_t grid = (n + 255) / 256;
+        if (grid > 65536) grid = 65536;
+        fp16_to_fp32_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(dst, src, n);
+        RLX_HIP(hipGetLastError());
+        return RLX_OK;
+    }
+    // measured on 2^28 elements (1.6 GB): 128 lanes x 4 elements 6.76 TB/s; 256 x 4, one or two rounds, 6.64 / 6.40;
+    // 64 x 4 x 2 6.58; 128 x 2 4.28 (too many workgroups for the dispatcher); one element per lane, grid-stride, 3.45
+    int lanes = 128, e = 4, rounds = 1;                           // variant 0
+    if (g_tuning.convert_variant == 1) e = 2;
+    else if (g_tuning.convert_variant == 3) { lanes = 256; rounds = 2; }
+    const int64_t span = (int64_t)lanes * e * rounds;
+    const int vec_ok = is_aligned(src, 2 * (size_t)e) && is_aligned(dst, 4 * (size_t)e);
+    const int64_t n_wg = (n + span - 1) / span;
+    for (int64_t first = 0; first < n_wg; first += kMaxTilesPerLaunch) {
+        const int64_t here = n_wg - first < kMaxTilesPerLaunch ? n_wg - first : kMaxTilesPerLaunch;
+        float* d = dst + first * span;
+        const uint16_t* q = src + first * span;
+        const int64_t left = n - first * span;
+        if (g_tuning.convert_variant == 1) convert_tile_kernel<128, 2, 1><<<dim3((unsigned)here), dim3(128), 0, s>>>(d, q, left, vec_ok);
+        else if (g_tuning.convert_variant == 3) convert_tile_kernel<256, 4, 2><<<dim3((unsigned)here), dim3(256), 0, s>>>(d, q, left, vec_ok);
+        else convert_tile_kernel<128, 4, 1><<<dim3((unsigned)here), dim3(128), 0, s>>>(d, q, left, vec_ok);
+        RLX_HIP(hipGetLastError());
+    }
     return RLX_OK;
 }
 
@@ -1025,8 +1413,7 @@ int rlx_scale_f32(float* x, float scale, int64_t n, void* stream) {
 int rlx_clear(void* dst, int64_t nbytes, void* stream) {
     if (nbytes <= 0) return RLX_OK;
     if (!dst) return RLX_ERR_INVALID_ARG;
-    clear_range(dst, nbytes, (hipStream_t)stream);
-    RLX_HIP(hipGetLastError());
+    RLX_HIP(clear_range(dst, nbytes, (hipStream_t)stream));
     return RLX_OK;
 }
 
@@ -1077,16 +1464,23 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
     p->n_tensors = count; p->n_chunks = n_chunks; p->n_elems = n_elems; p->chunk_elems = chunk_elems;
     p->any_master = false;
     p->idle_by_range = true;
+    try {
+        p->idle_grads.reserve(kMaxIdleRanges);
+    } catch (const std::bad_alloc&) {
+        delete p;
+        return RLX_ERR_NO_MEMORY;
+    }
     for (int64_t i = 0; i < count; i++) {
         p->any_master = p->any_master || descs[i].master != nullptr;
         if (descs[i].flags & (RLX_TENSOR_GRAD_ONLY | RLX_TENSOR_FROZEN)) {
-            if (p->idle_grads.size() < kMaxIdleRanges)
+            if (p->idle_grads.size() < kMaxIdleRanges)      // within the reserved capacity: cannot throw
                 p->idle_grads.emplace_back(descs[i].grad, descs[i].n * (descs[i].dtype == RLX_DTYPE_F16 ? 2 : 4));
             else
                 p->idle_by_range = false;
         }
     }
     p->d_recs = nullptr; p->d_active = nullptr; p->n_active = 0; p->d_partials = nullptr; p->d_norm = nullptr; p->h_norm = nullptr;
+    p->d_sched = nullptr; p->sched_cap = 0; p->sched_len = 0; p->d_current = nullptr; p->d_taken = nullptr;
 
     hipError_t e = hipGetDevice(&p->device);
     if (e == hipSuccess) e = hipMalloc((void**)&p->d_recs, sizeof(ChunkRec) * (size_t)n_chunks);
@@ -1133,6 +1527,8 @@ int rlx_plan_destroy(rlx_plan* p) {
     if (p->d_partials && (e = hipFree(p->d_partials)) != hipSuccess && first == hipSuccess) first = e;
     if (p->d_norm && (e = hipFree(p->d_norm)) != hipSuccess && first == hipSuccess) first = e;
     if (p->h_norm && (e = hipHostFree(p->h_norm)) != hipSuccess && first == hipSuccess) first = e;
+    if (p->d_sched && (e = hipFree(p->d_sched)) != hipSuccess && first == hipSuccess) first = e;
+    if (p->d_current && (e = hipFree(p->d_current)) != hipSuccess && first == hipSuccess) first = e;
     p->magic = 0;
     delete p;
     return first == hipSuccess ? RLX_OK : hip_fail(first, "rlx_plan_destroy");
@@ -1195,8 +1591,7 @@ int rlx_grad_norm_static(const uint16_t* half_grads, int64_t n_half, const float
     const int st = static_scratch(&partials);
     if (st != RLX_OK) return st;
     if (n_chunks == 0) {      // nothing to add up: sum 0, norm 0, scale by the rule
-        sumsq_final_kernel<<<dim3(1), dim3(kFinalBlock), 0, (hipStream_t)stream>>>(partials, 0, max_norm,
-                                                                                   (NormResult*)result_dev);
+        launch_final(partials, 0, max_norm, (NormResult*)result_dev, (hipStream_t)stream);
         RLX_HIP(hipGetLastError());
         return RLX_OK;
     }
@@ -1248,6 +1643,67 @@ int rlx_plan_adamw_dev(rlx_plan* p, const rlx_step_params* dev_params, int step_
     return plan_update(p, h, dev_params, step_flags, (hipStream_t)stream);
 }
 
+int rlx_plan_schedule_upload(rlx_plan* p, const rlx_step_params* steps, int64_t n_steps, void* stream) {
+    if (!plan_ok(p) || !steps || n_steps <= 0 || n_steps > ((int64_t)1 << 28)) return RLX_ERR_INVALID_ARG;
+    const int ready = plan_launchable(p);
+    if (ready != RLX_OK) return ready;
+    for (int64_t i = 0; i < n_steps; i++) {
+        const int st = check_hyper(steps[i].lr, steps[i].beta1, steps[i].beta2, steps[i].eps, steps[i].weight_decay,
+                                   steps[i].bias_correction1, steps[i].bias_correction2);
+        if (st != RLX_OK) return st;
+    }
+    // scheduled updates already in the stream still read the old table
+    RLX_HIP(hipStreamSynchronize((hipStream_t)stream));
+    if (!p->d_current) {
+        // one small allocation: the current entry (28 bytes, padded to 32) followed by the step count
+        RLX_HIP(hipMalloc((void**)&p->d_current, 40));
+        p->d_taken = (int64_t*)((char*)p->d_current + 32);
+    }
+    if (n_steps > p->sched_cap) {
+        if (p->d_sched) RLX_HIP(hipFree(p->d_sched));
+        p->d_sched = nullptr; p->sched_cap = 0;
+        RLX_HIP(hipMalloc((void**)&p->d_sched, sizeof(rlx_step_params) * (size_t)n_steps));
+        p->sched_cap = n_steps;
+    }
+    const int64_t zero = 0;
+    RLX_HIP(hipMemcpy(p->d_sched, steps, sizeof(rlx_step_params) * (size_t)n_steps, hipMemcpyHostToDevice));
+    RLX_HIP(hipMemcpy(p->d_current, steps, sizeof(rlx_step_params), hipMemcpyHostToDevice));
+    RLX_HIP(hipMemcpy(p->d_taken, &zero, sizeof(zero), hipMemcpyHostToDevice));
+    p->sched_len = n_steps;
+    return RLX_OK;
+}
+
+int rlx_plan_adamw_scheduled(rlx_plan* p, int step_flags, void* stream) {
+    if (!plan_ok(p) || !p->d_sched || p->sched_len <= 0) return RLX_ERR_INVALID_ARG;
+    if (step_flags & ~(RLX_CLIP_FUSED | RLX_STEP_ZERO_GRADS)) return RLX_ERR_INVALID_ARG;
+    const int ready = plan_launchable(p);
+    if (ready != RLX_OK) return ready;
+    Hyper h;
+    memset(&h, 0, sizeof(h));
+    const int st = plan_update(p, h, p->d_current, step_flags, (hipStream_t)stream);
+    if (st != RLX_OK) return st;
+    schedule_advance_kernel<<<dim3(1), dim3(64), 0, (hipStream_t)stream>>>(p->d_sched, p->sched_len, p->d_taken,
+                                                                          p->d_current);
+    RLX_HIP(hipGetLastError());
+    return RLX_OK;
+}
+
+int rlx_plan_schedule_position(rlx_plan* p, int64_t* steps_taken, int64_t* n_steps, void* stream) {
+    if (!plan_ok(p) || !p->d_sched) return RLX_ERR_INVALID_ARG;
+    const int ready = plan_launchable(p);
+    if (ready != RLX_OK) return ready;
+    int64_t taken = 0;
+    RLX_HIP(hipStreamSynchronize((hipStream_t)stream));
+    RLX_HIP(hipMemcpy(&taken, p->d_taken, sizeof(taken), hipMemcpyDeviceToHost));
+    if (steps_taken) *steps_taken = taken;
+    if (n_steps) *n_steps = p->sched_len;
+    return RLX_OK;
+}
+
+const char* rlx_update_variant_name(int64_t variant) {
+    return variant >= 0 && variant < kNumUpdateVariants ? kVariantNames[variant] : "";
+}
+
 int rlx_set_tuning(const char* key, int64_t value) {
     if (!key || value < 0) return RLX_ERR_INVALID_ARG;
     if (!strcmp(key, "update_variant")) {
@@ -1255,7 +1711,15 @@ int rlx_set_tuning(const char* key, int64_t value) {
         g_tuning.update_variant = value;
     } else if (!strcmp(key, "norm_grid")) g_tuning.norm_grid = value;
     else if (!strcmp(key, "norm_nt")) g_tuning.norm_nt = value ? 1 : 0;
-    else return RLX_ERR_INVALID_ARG;
+    else if (!strcmp(key, "norm_pack")) {
+        if (value > 3) return RLX_ERR_INVALID_ARG;
+        g_tuning.norm_pack = value;
+    }
+    else if (!strcmp(key, "final_batch")) g_tuning.final_batch = value;
+    else if (!strcmp(key, "convert_variant")) {
+        if (value >= kNumConvertVariants) return RLX_ERR_INVALID_ARG;
+        g_tuning.convert_variant = value;
+    } else return RLX_ERR_INVALID_ARG;
     return RLX_OK;
 }
 
@@ -1264,6 +1728,9 @@ int64_t rlx_get_tuning(const char* key) {
     if (!strcmp(key, "update_variant")) return g_tuning.update_variant;
     if (!strcmp(key, "norm_grid")) return g_tuning.norm_grid;
     if (!strcmp(key, "norm_nt")) return g_tuning.norm_nt;
+    if (!strcmp(key, "norm_pack")) return g_tuning.norm_pack;
+    if (!strcmp(key, "convert_variant")) return g_tuning.convert_variant;
+    if (!strcmp(key, "final_batch")) return g_tuning.final_batch;
     return -1;
 }
 

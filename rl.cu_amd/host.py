@@ -196,6 +196,28 @@ class AdamWOptimizer:
         flags = (B.CLIP_FUSED if fused_clip else 0) | (B.STEP_ZERO_GRADS if zero_grads else 0)
         self.plan.adamw(self.step_params(), flags, _stream() if stream is None else stream)
 
+    # --- steps without the host (a recorded norm + update replayed step after step) ----------------------
+    def upload_schedule(self, lrs, stream=None):
+        """Uploads the hyper-parameters of the next len(lrs) steps (steps get_step()+1, ...): the given learning
+        rates (from the LR scheduler) and the bias corrections 1 - powf(beta, t) computed here on the host, as
+        optimizer.h:120-122 computes them.  Blocking; call outside the step loop."""
+        steps = [B.StepParams(lr, self.beta1, self.beta2, self.eps, self.weight_decay,
+                              bias_correction(self.beta1, self.step_ + 1 + k),
+                              bias_correction(self.beta2, self.step_ + 1 + k)) for k, lr in enumerate(lrs)]
+        self.plan.schedule_upload(steps, _stream() if stream is None else stream)
+        self._scheduled_lrs = list(lrs)
+        self._scheduled_from = self.step_
+
+    def step_scheduled(self, fused_clip=False, zero_grads=False, stream=None):
+        """step() with the hyper-parameters of the uploaded table; the device moves on to the next entry by
+        itself, so a captured launch can be replayed without any host write in between."""
+        k = self.step_ - self._scheduled_from
+        if 0 <= k < len(self._scheduled_lrs):
+            self.lr = self._scheduled_lrs[k]           # host-side bookkeeping only; the device reads its table
+        self.step_ += 1
+        flags = (B.CLIP_FUSED if fused_clip else 0) | (B.STEP_ZERO_GRADS if zero_grads else 0)
+        self.plan.adamw_scheduled(flags, _stream() if stream is None else stream)
+
     # --- optimizer state on disk (the reference's save_checkpoint is a stub, trainer.h:317-319) ----
     # One format, shared with the C++ AdamWOptimizer (rl.cu_amd/host/training/optimizer.h): "RLXOPT02", int32
     # step, 5 x float32 (lr, beta1, beta2, eps, weight_decay), int32 sections; per section uint16 name length,

@@ -244,6 +244,32 @@ public:
         RLX_CHECK(rlx_plan_adamw(plan_for(grads), &sp, flags, (void*)stream));
     }
 
+    // Steps without the host (a recorded norm + update replayed step after step).  upload_schedule puts the
+    // hyper-parameters of the next n steps (steps get_step()+1, ...) on the device: the given learning rates and
+    // the bias corrections formed here with powf, as in step().  step_scheduled launches the update with the
+    // current entry; the device then moves on to the next entry by itself, so a captured step_scheduled can be
+    // replayed with nothing written by the host in between (advance get_step() with note_replayed_steps).
+    template <class Grads>
+    void upload_schedule(Grads* grads, const float* lrs, int n, hipStream_t stream = 0) {
+        std::vector<rlx_step_params> steps((size_t)n);
+        for (int k = 0; k < n; k++) {
+            rlx_step_params& sp = steps[(size_t)k];
+            sp.lr = lrs[k]; sp.beta1 = beta1; sp.beta2 = beta2; sp.eps = eps; sp.weight_decay = weight_decay;
+            sp.bias_correction1 = 1.0f - powf(beta1, (float)(step_ + 1 + k));
+            sp.bias_correction2 = 1.0f - powf(beta2, (float)(step_ + 1 + k));
+        }
+        RLX_CHECK(rlx_plan_schedule_upload(plan_for(grads), steps.data(), n, (void*)stream));
+    }
+    template <class Grads>
+    void step_scheduled(Grads* grads, hipStream_t stream = 0) {
+        const bool fused = clip_pending_;
+        clip_pending_ = false;
+        step_++;
+        const int flags = (fused ? RLX_CLIP_FUSED : 0) | (zero_grads_ ? RLX_STEP_ZERO_GRADS : 0);
+        RLX_CHECK(rlx_plan_adamw_scheduled(plan_for(grads), flags, (void*)stream));
+    }
+    void note_replayed_steps(int n) { step_ += n; }
+
     // Trainer::clip_grad_norm_ (trainer.h:323-352) over the same gradient type: clips all gradients
     // (half_pool + float_pool) so that the global L2 norm is <= max_norm and returns the pre-clip norm
     // (host scalar, synchronous), like the reference.  With set_fused_clip(true) the gradients stay as they

@@ -93,6 +93,19 @@ def test_plan_argument_checks(B):
     assert lib.rlx_plan_grad_norm(None, 1.0, None) == B.ERR_INVALID_ARG
     assert lib.rlx_plan_adamw(None, None, 0, None) == B.ERR_INVALID_ARG
     assert lib.rlx_plan_adamw_dev(None, None, 0, None) == B.ERR_INVALID_ARG
+    sp = (B.StepParams * 1)(B.StepParams(1e-3, 0.9, 0.999, 1e-8, 0.0, 0.1, 0.001))
+    assert lib.rlx_plan_schedule_upload(None, sp, 1, None) == B.ERR_INVALID_ARG
+    assert lib.rlx_plan_adamw_scheduled(None, 0, None) == B.ERR_INVALID_ARG
+    assert lib.rlx_plan_schedule_position(None, None, None, None) == B.ERR_INVALID_ARG
+    # the entry point that allocates nothing checks its arguments before it touches a device
+    assert B.grad_norm_static(0x1000, -1, None, 0, 1.0, 0x2000) == B.ERR_INVALID_ARG
+    assert B.grad_norm_static(None, 8, None, 0, 1.0, 0x2000) == B.ERR_INVALID_ARG
+    assert B.grad_norm_static(0x1000, 8, None, 0, 1.0, None) == B.ERR_INVALID_ARG
+    assert B.grad_norm_static(0x1001, 8, None, 0, 1.0, 0x2000) == B.ERR_MISALIGNED
+    assert B.grad_norm_static(0x1000, 8, 0x3002, 8, 1.0, 0x2000) == B.ERR_MISALIGNED
+    assert B.grad_norm_static(0x1000, 8, None, 0, 1.0, 0x2004) == B.ERR_MISALIGNED
+    assert B.grad_norm_static(0x1000, 8, None, 0, 1.0, 0x2000, chunk_elems=1000) == B.ERR_INVALID_ARG
+    assert B.grad_norm_static(0x1000, (1 << 18) * 512 + 1, None, 0, 1.0, 0x2000, chunk_elems=512) == B.ERR_TOO_LARGE
 
 
 def test_tuning_keys(B):
@@ -105,6 +118,18 @@ def test_tuning_keys(B):
     with pytest.raises(B.RlxError):
         B.set_tuning("no_such_key", 1)
     assert B.get_tuning("no_such_key") == -1
+    for key, top in (("norm_pack", 3), ("convert_variant", 3), ("final_batch", 40)):
+        default = B.get_tuning(key)
+        B.set_tuning(key, top)
+        assert B.get_tuning(key) == top
+        B.set_tuning(key, default)
+    with pytest.raises(B.RlxError):
+        B.set_tuning("convert_variant", 4)
+    # every update variant has a kernel name; the default names the shipped tile shape
+    names = [B.update_variant_name(v) for v in range(15)]
+    assert all(names) and len(set(names)) == 15 and B.update_variant_name(15) == ""
+    assert names[0].startswith("adamw_tile_kernel<2,128,1,") and B.update_variant_name() == names[0]
+    assert "persistent" in names[11] and "chunk" in names[12]
 
 
 def test_layouts(L):

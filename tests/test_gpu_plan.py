@@ -288,16 +288,18 @@ def test_ragged_list_equals_flat_tensor(O, L, host, B, torch_gpu):
 
 @pytest.mark.parametrize("master,zero_grads", [(False, False), (True, False), (False, True), (True, True)])
 def test_every_tile_shape_and_chunk_size_gives_the_same_bits(L, host, B, torch_gpu, master, zero_grads):
-    """Every compiled form of the update kernel (tile shapes, XCD swizzle, store policy, and the two forms that
-    issue their loads and stores at once or two at a time) gives the same bits, with and without a master copy
-    and gradient clearing (which select between those two forms by default)."""
+    """Every compiled form of the update kernel (tile shapes, XCD swizzle, store policy, the two forms that
+    issue their loads and stores at once or two at a time, and the 128-bit-access forms: one wavefront per tile,
+    a persistent grid striding over the tiles, one workgroup walking a chunk) gives the same bits, with and
+    without a master copy and gradient clearing (which select between the first two forms by default)."""
     torch = torch_gpu
     specs = [L.TensorSpec("a", 70_001, L.DTYPE_F16, 0, 0), L.TensorSpec("b", 2049, L.DTYPE_F32, 0, 0),
              L.TensorSpec("c", 131, L.DTYPE_F16, L.NO_DECAY, 0)]
     results = []
     try:
         for variant, chunk in [(0, 8192), (1, 8192), (2, 2048), (3, 512), (4, 512), (5, 65536), (6, 1024),
-                               (7, 2048), (8, 8192), (9, 4096)]:
+                               (7, 2048), (8, 8192), (9, 4096), (10, 512), (10, 8192), (11, 512), (11, 2048),
+                               (11, 65536), (12, 512), (12, 8192), (13, 2048), (14, 8192)]:
             B.set_tuning("update_variant", variant)
             st = host.ParamStore(specs, master=master)
             st.fill("p", 1, 0.0, 0.02)
@@ -438,6 +440,155 @@ def test_device_resident_step_params_and_graph_replay(O, L, host, B, torch_gpu):
         assert sum_sq == O.sumsq_mirror([h["g"] for h in hs], 2048)[0]
         oracle_step(O, L, specs, hs, step, dict(HYPER, lr=lr), clip_scale=scale)
         assert compare(st, hs, "replay %d" % step) == 0
+
+
+def test_scheduled_steps_replay_without_the_host(O, L, host, B, torch_gpu):
+    """norm + fused-clip update + advance recorded once as a HIP graph; the hyper-parameters of six steps (a
+    decaying learning rate, host-computed bias corrections) are uploaded once, and the graph is replayed five
+    times with NO host write of hyper-parameters in between: only new gradients arrive (eager fills and
+    synchronisations between the replays).  Every replay equals the oracle; the sixth, eager, scheduled step
+    uses the sixth entry; a seventh reuses it (the table is exhausted) and the position saturates."""
+    torch = torch_gpu
+    specs = L.qwen3_tensor_list(MINI, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
+    st = host.ParamStore(specs)
+    st.fill("p", 1, 0.0, 0.02)
+    st.fill("g", 2, 0.0, 5e-3)
+    opt = host.AdamWOptimizer(st, lr=1e-3, chunk_elems=2048)
+    torch.cuda.synchronize()
+    hs = host_copy(st)
+    lrs = [1e-3 / k for k in range(1, 7)]
+    # a table with a zero bias correction or a non-finite rate is refused and changes nothing
+    bad = [B.StepParams(1e-3, 0.9, 0.999, 1e-8, 0.01, 0.1, 0.0)]
+    with pytest.raises(B.RlxError) as err:
+        opt.plan.schedule_upload(bad)
+    assert err.value.status == B.ERR_BAD_HYPER
+    with pytest.raises(B.RlxError):
+        opt.plan.adamw_scheduled()                               # no table yet
+    opt.upload_schedule(lrs)
+    assert opt.plan.schedule_position() == (0, 6)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            s = torch.cuda.current_stream().cuda_stream
+            opt.plan.grad_norm(0.5, s)
+            opt.plan.adamw_scheduled(B.CLIP_FUSED, s)
+    torch.cuda.synchronize()
+    assert opt.plan.schedule_position() == (0, 6)                # capturing ran nothing
+
+    def check(step, lr):
+        norm, scale, sum_sq = opt.plan.norm_read()
+        assert sum_sq == O.sumsq_mirror([h["g"] for h in hs], 2048)[0] and norm > 0.5
+        oracle_step(O, L, specs, hs, step, dict(HYPER, lr=lr), clip_scale=scale)
+        assert compare(st, hs, "scheduled step %d" % step) == 0
+
+    for step in range(1, 6):
+        if step > 1:
+            st.fill("g", 2 + step, 0.0, 5e-3 * step)             # new gradients: the only thing the host provides
+            torch.cuda.synchronize()
+            for i, h in enumerate(hs):
+                h["g"] = bits(st.grad(i))
+        graph.replay()
+        torch.cuda.synchronize()
+        check(step, lrs[step - 1])
+        assert opt.plan.schedule_position() == (step, 6)
+    # eager scheduled steps continue where the replays left off
+    opt.step_ = 5
+    for step, lr in ((6, lrs[5]), (7, lrs[5])):
+        opt.plan.grad_norm(0.5)
+        opt.step_scheduled(fused_clip=True)
+        torch.cuda.synchronize()
+        if step == 6:
+            check(6, lr)
+            assert opt.plan.schedule_position() == (6, 6)
+        else:
+            # exhausted: the last entry (step 6's bias corrections and rate) is used again
+            norm, scale, _ = opt.plan.norm_read()
+            bc1, bc2 = O.bias_correction(0.9, 6), O.bias_correction(0.999, 6)
+            for s_, h in zip(specs, hs):
+                wd = 0.0 if s_.flags & L.NO_DECAY else 0.01
+                fn = O.adamw_fp16 if s_.dtype == L.DTYPE_F16 else O.adamw_fp32
+                args = (None,) if s_.dtype == L.DTYPE_F16 else ()
+                fn(*args, h["p"], h["g"], h["m"], h["v"], lr, 0.9, 0.999, 1e-8, wd, bc1, bc2, clip_scale=scale)
+            assert compare(st, hs, "step beyond the table") == 0
+            assert opt.plan.schedule_position() == (6, 6)
+    # a new upload starts again at its first entry
+    opt.upload_schedule([2e-4])
+    assert opt.plan.schedule_position() == (0, 1)
+
+
+def test_packed_norm_pass_gives_the_same_partials(O, L, host, B, torch_gpu):
+    """512-element chunks: the forms of the first pass that give a workgroup 32, 16, 8 or one chunk, and every
+    load depth of the second pass, write the same per-chunk partials and the same result, equal to the
+    restated order; FP32 tensors, sizes that are no multiple of 8, and a frozen tensor included."""
+    torch = torch_gpu
+    specs = L.ragged_tensor_list(count=300, seed=11)
+    specs += [L.TensorSpec("f32.%d" % i, n, L.DTYPE_F32, 0, 0) for i, n in enumerate((1, 3, 4, 5, 8, 509, 512, 513, 1027))]
+    specs += [L.TensorSpec("frozen", 700, L.DTYPE_F16, L.FROZEN, 0)]
+    st = host.ParamStore(specs)
+    st.fill("g", 7, 0.0, 3e-3)
+    opt = host.AdamWOptimizer(st, lr=1e-3, chunk_elems=512)
+    torch.cuda.synchronize()
+    grads = [bits(st.grad(i)) for i in range(len(specs))]
+    grads[-1] = np.zeros_like(grads[-1])                         # a frozen tensor's gradients count as zero
+    want, parts = O.sumsq_mirror(grads, 512)
+    got = {}
+    try:
+        for pack, batch in ((2, 16), (3, 8), (1, 32), (0, 40)):
+            B.set_tuning("norm_pack", pack)
+            B.set_tuning("final_batch", batch)
+            opt.plan.grad_norm(1.0)
+            _, _, sum_sq = opt.plan.norm_read()
+            got[pack] = (sum_sq, read_device(opt.plan.partials_ptr, 8 * opt.plan.num_chunks).view(np.float64).copy())
+    finally:
+        B.set_tuning("norm_pack", 2)
+        B.set_tuning("final_batch", 0)
+    for pack in got:
+        assert got[pack][0] == want, pack
+        assert np.array_equal(got[pack][1], parts), pack
+
+
+@pytest.mark.parametrize("n,src_off,dst_off", [(1 << 20, 0, 0), (2048 * 5 + 777, 0, 0), (300_001, 1, 0), (300_001, 0, 1),
+                                               (4097, 4, 4), (100, 0, 0), (2048, 2, 2)])
+def test_fp16_to_fp32_every_form(O, B, torch_gpu, n, src_off, dst_off):
+    """The master-copy initialisation dst[i] = (float)src[i] (optimizer.h:46-57) in its four compiled forms, for
+    whole and ragged sizes and for starts that are not aligned for the wide accesses: identical to the oracle's
+    conversion, and nothing written outside [dst, dst + n)."""
+    torch = torch_gpu
+    src = torch.empty(n + 16, dtype=torch.float16, device="cuda:0")
+    B.fill_f16(src.data_ptr(), n + 16, 31, 0.0, 3.0)
+    want = O.h2f(bits(src)[src_off: src_off + n])
+    try:
+        for variant in (0, 1, 2, 3):
+            B.set_tuning("convert_variant", variant)
+            dst = torch.full((n + 16,), -7.0, dtype=torch.float32, device="cuda:0")
+            assert B.fp16_to_fp32(dst.data_ptr() + 4 * dst_off, src.data_ptr() + 2 * src_off, n) == B.OK
+            torch.cuda.synchronize()
+            out = dst.cpu().numpy()
+            assert np.array_equal(out[dst_off: dst_off + n].view(np.uint32), want.view(np.uint32)), variant
+            assert (out[:dst_off] == -7.0).all() and (out[dst_off + n:] == -7.0).all(), variant
+    finally:
+        B.set_tuning("convert_variant", 0)
+
+
+def test_plan_launches_on_its_own_device_after_a_device_round_trip(B, torch_gpu):
+    """The device check that guards every plan launch (RLX_ERR_WRONG_DEVICE when another device is current) lets
+    the owning device through, also after the current device has been set again explicitly."""
+    torch = torch_gpu
+    n = 4096
+    p = torch.zeros(n, dtype=torch.float16, device="cuda:0"); g = torch.ones_like(p)
+    m = torch.zeros(n, dtype=torch.float32, device="cuda:0"); v = torch.zeros_like(m)
+    plan = B.Plan([B.TensorDesc(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), None, n, B.DTYPE_F16, 0)])
+    lib = B.load()
+    sp = B.StepParams(1e-3, 0.9, 0.999, 1e-8, 0.0, 0.1, 0.001)
+    torch.cuda.set_device(0)
+    with torch.cuda.device(0):
+        assert lib.rlx_plan_grad_norm(plan._h, 1.0, None) == B.OK
+        assert lib.rlx_plan_adamw(plan._h, sp, B.CLIP_FUSED, None) == B.OK
+        assert lib.rlx_plan_scale_grads(plan._h, None) == B.OK
+    torch.cuda.synchronize()
+    assert plan.norm_read()[0] == 64.0                           # sqrt(4096 ones)
+    assert lib.rlx_status_string(B.ERR_WRONG_DEVICE) == b"the plan belongs to another device than the current one"
 
 
 def test_clip_rounds_twice_for_every_half_and_many_scales(O, L, host, B, torch_gpu):
