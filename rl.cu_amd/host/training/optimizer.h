@@ -294,6 +294,9 @@ public:
     // fp32.v.  Data moves through a 64 MB staging buffer, so the host never holds a whole pool.
     // Both return false (and print why) on failure; load_state checks the whole file before it touches the
     // state and leaves it alone if anything is wrong.
+    // Size of the staging buffer of save_state / load_state in floats (default 16 Mi = 64 MB).
+    void set_state_staging(size_t floats) { stage_limit_ = floats ? floats : 1; }
+
     bool save_state(const std::string& path) const {
         HIP_CHECK(hipDeviceSynchronize());
         const std::string tmp = path + ".tmp";
@@ -472,11 +475,11 @@ private:
         return s;
     }
     static constexpr const char* kStateMagic = "RLXOPT02";
-    static constexpr size_t kStageFloats = (size_t)16 << 20;         // 64 MB between the device and the file
-    static size_t stage_floats(const std::vector<Section>& secs) {
+    size_t stage_limit_ = (size_t)16 << 20;         // floats: 64 MB between the device and the file
+    size_t stage_floats(const std::vector<Section>& secs) const {
         size_t most = 1;
         for (const Section& s : secs) most = s.n > most ? s.n : most;
-        return most < kStageFloats ? most : kStageFloats;
+        return most < stage_limit_ ? most : stage_limit_;
     }
     static uint64_t word_sum(const float* p, size_t n) {
         uint64_t acc = 0;
@@ -530,7 +533,7 @@ private:
         fp16_state_ = o.fp16_state_; fp32_state_ = o.fp32_state_;
         n16_ = o.n16_; n32_ = o.n32_; proj_n_ = o.proj_n_;
         plan_ = o.plan_; plan_half_ = o.plan_half_; plan_float_ = o.plan_float_; plan_float_bytes_ = o.plan_float_bytes_;
-        embed_frozen_ = o.embed_frozen_;
+        embed_frozen_ = o.embed_frozen_; stage_limit_ = o.stage_limit_;
         fused_clip_ = o.fused_clip_; zero_grads_ = o.zero_grads_; clip_pending_ = o.clip_pending_;
         o.plan_ = nullptr; o.fp16_state_ = nullptr; o.fp32_state_ = nullptr;
         o.fp16_master_ = o.fp16_m_ = o.fp16_v_ = o.fp32_m_ = o.fp32_v_ = nullptr;

@@ -11,6 +11,7 @@
 //   6. operator API (launch_adamw_fp16 / launch_adamw_fp32) on raw pointers
 //   7. frozen embedding flagged in the plan, gradients cleared inside the update
 //   8. optimizer state save / load   9. train loop with LR schedule and JSON-lines log
+//   10. gradient pools   11. training_step with accumulation   12. steps from an uploaded table of hyper-parameters
 // The oracle (liborc_adamw.so) is used as the checker only.
 #include <cmath>
 #include <cstdint>
@@ -286,6 +287,8 @@ static void test_checkpoint() {
     AdamWOptimizer oa(a.pools, 1e-3f), ob(b.pools, 1e-3f);
     OptimStepConfig c; c.max_grad_norm = 0.25f; c.fused_clip = true;
     OptimStep sa(&oa, c), sb(&ob, c);
+    oa.set_state_staging(10000);      // sections of 57,600 and 2,368 floats pass through a 10,000-float buffer
+    ob.set_state_staging(777);
     for (int i = 0; i < 3; i++) sa.apply(&a.grads);
     bool ok = oa.save_state(path);
     HIP_CHECK(hipMemcpy(b.w16, a.w16, a.n16 * 2, hipMemcpyDeviceToDevice));   // weights are the model's to save
@@ -447,6 +450,44 @@ static void test_accumulation() {
     else FAIL(name, "scaled=%d loss=%f na=%f nb=%f diff=%zu", scaled, loss, sa.last_grad_norm(), nb, diff);
 }
 
+// 12. Steps from an uploaded table of hyper-parameters (no host values at launch time) equal ordinary steps
+//     with set_lr: rates from the LR scheduler, bias corrections formed by the same powf
+static void test_scheduled_steps() {
+    const char* name = "scheduled steps == set_lr + step";
+    Fixture a(5e-3f), b(5e-3f);
+    AdamWOptimizer oa(a.pools, 1e-3f), ob(b.pools, 1e-3f);
+    oa.set_fused_clip(true); ob.set_fused_clip(true);
+    LRScheduler sched;
+    sched.init_cosine(1e-3f, 1e-4f, 1, 6);
+    float lrs[4];
+    for (int k = 0; k < 4; k++) lrs[k] = sched.get_lr(k);
+    ob.upload_schedule(&b.grads, lrs, 4);
+    bool ok = true;
+    for (int k = 0; k < 4; k++) {
+        oa.set_lr(lrs[k]);
+        const float na = oa.clip_grad_norm_(&a.grads, 0.25f);
+        oa.step(&a.grads);
+        const float nb = ob.clip_grad_norm_(&b.grads, 0.25f);
+        ob.step_scheduled(&b.grads);
+        ok = ok && na == nb;
+    }
+    HIP_CHECK(hipDeviceSynchronize());
+    int64_t taken = -1, total = -1;
+    RLX_CHECK(rlx_plan_schedule_position(ob.plan_for(&b.grads), &taken, &total, nullptr));
+    a.download(); b.download();
+    size_t diff = 0;
+    for (size_t i = 0; i < a.n16; i++) diff += a.h_w16[i] != b.h_w16[i];
+    for (size_t i = 0; i < a.n32; i++) diff += memcmp(&a.h_w32[i], &b.h_w32[i], 4) != 0;
+    auto ma = d2h(oa.fp16_master(), a.n16), mb = d2h(ob.fp16_master(), b.n16);
+    auto va = d2h(oa.fp16_v(), a.n16), vb = d2h(ob.fp16_v(), b.n16);
+    for (size_t i = 0; i < a.n16; i++) diff += memcmp(&ma[i], &mb[i], 4) != 0 || memcmp(&va[i], &vb[i], 4) != 0;
+    // a table with a zero bias correction is refused
+    rlx_step_params bad = {1e-3f, 0.9f, 0.999f, 1e-8f, 0.0f, 0.0f, 0.1f};
+    const bool refused = rlx_plan_schedule_upload(ob.plan_for(&b.grads), &bad, 1, nullptr) == RLX_ERR_BAD_HYPER;
+    if (ok && diff == 0 && taken == 4 && total == 4 && refused && ob.get_step() == 4) PASS(name);
+    else FAIL(name, "ok=%d diff=%zu taken=%lld total=%lld refused=%d", ok, diff, (long long)taken, (long long)total, refused);
+}
+
 int main() {
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
@@ -465,6 +506,7 @@ int main() {
     test_train_loop();
     test_grad_pools();
     test_accumulation();
+    test_scheduled_steps();
     printf("=== %s (%d failure%s) ===\n", g_fails ? "FAILED" : "ALL PASSED", g_fails, g_fails == 1 ? "" : "s");
     return g_fails;
 }

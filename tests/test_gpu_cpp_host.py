@@ -18,7 +18,7 @@ def test_cpp_host_mirror(torch_gpu):
     print(res.stdout)
     print(res.stderr)
     assert res.returncode == 0, res.stdout + res.stderr
-    assert res.stdout.count("[PASS]") == 11 and "[FAIL]" not in res.stdout
+    assert res.stdout.count("[PASS]") == 12 and "[FAIL]" not in res.stdout
 
 
 def test_reference_call_sites_compile_unchanged_and_match_the_oracle(torch_gpu):

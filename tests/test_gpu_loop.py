@@ -35,6 +35,8 @@ def test_checkpoint_resume_is_bit_identical(L, host, torch_gpu, tmp_path, master
         st_a.fill("g", 10 + step, 0.0, 5e-3)
         host.training_step(opt_a, 0.5, fused_clip=True)
     path = str(tmp_path / "opt.state")
+    if master:
+        opt_a.CKPT_STAGE = 1000                  # every tensor passes through the staging buffer in several pieces
     opt_a.save_state(path)
     weights = [st_a.p16.clone(), st_a.p32.clone()]
     for step in range(4, 6):
@@ -44,6 +46,8 @@ def test_checkpoint_resume_is_bit_identical(L, host, torch_gpu, tmp_path, master
     _, st_b, opt_b = make(L, host, master)
     st_b.p16.copy_(weights[0])
     st_b.p32.copy_(weights[1])
+    if master:
+        opt_b.CKPT_STAGE = 333
     opt_b.load_state(path)
     assert opt_b.get_step() == 3 and abs(opt_b.lr - 1e-3) < 1e-9
     for step in range(4, 6):
