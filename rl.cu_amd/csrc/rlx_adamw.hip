@@ -31,6 +31,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <atomic>
 #include <cstring>
 #include <mutex>
 #include <new>
@@ -938,14 +939,16 @@ int hip_fail(hipError_t e, const char* what) {
         if (e_ != hipSuccess) return hip_fail(e_, #call);    \
     } while (0)
 
+// Process-wide launch tuning (for measurement).  Atomic, so that a thread that changes a key while another
+// launches is a defined race: every launch reads each key once and uses one consistent choice.
 struct Tuning {
-    int64_t update_variant = 0;
-    int64_t norm_grid = 0;
-    int64_t norm_nt = 1;
-    int64_t norm_pack = 2;          // 512-element chunks per workgroup: 0 = one, 1 = eight (a wavefront each),
-                                    // 2 = thirty-two (four per wavefront, the default), 3 = sixteen
-    int64_t convert_variant = 0;
-    int64_t final_batch = 0;        // loads in flight per lane in the second pass of the norm; 0 = by the number of partials
+    std::atomic<int64_t> update_variant{0};
+    std::atomic<int64_t> norm_grid{0};
+    std::atomic<int64_t> norm_nt{1};
+    std::atomic<int64_t> norm_pack{2};      // 512-element chunks per workgroup: 0 = one, 1 = eight (a wavefront each),
+                                            // 2 = thirty-two (four per wavefront, the default), 3 = sixteen
+    std::atomic<int64_t> convert_variant{0};
+    std::atomic<int64_t> final_batch{0};    // loads in flight per lane in the second pass of the norm; 0 = by the number of partials
 } g_tuning;
 
 constexpr int kNumUpdateVariants = 15;
@@ -1257,14 +1260,16 @@ void launch_final(const double* partials, int64_t n, float max_norm, NormResult*
 template <bool POOLS>
 int launch_norm(const ChunkRec* recs, const PoolPair& pools, int64_t n_chunks, int64_t chunk_elems, double* partials,
                 float max_norm, NormResult* result, hipStream_t s) {
-    int64_t g = g_tuning.norm_grid > 0 ? g_tuning.norm_grid : n_chunks;
+    const int64_t norm_grid = g_tuning.norm_grid, norm_pack = g_tuning.norm_pack;
+    const bool norm_nt = g_tuning.norm_nt != 0;
+    int64_t g = norm_grid > 0 ? norm_grid : n_chunks;
     if (g > n_chunks) g = n_chunks;
     if (g > kMaxNormGrid) g = kMaxNormGrid;
     const dim3 grid((unsigned)g);
     const int64_t lanes = chunk_elems / kVec < kNormBlock ? chunk_elems / kVec : kNormBlock;
 #define RLX_NORM_LAUNCH(BLOCK)                                                                                       \
     do {                                                                                                             \
-        if (g_tuning.norm_nt)                                                                                        \
+        if (norm_nt)                                                                                        \
             sumsq_partials_kernel<true, BLOCK, POOLS><<<grid, dim3(BLOCK), 0, s>>>(recs, pools, n_chunks, partials);  \
         else                                                                                                         \
             sumsq_partials_kernel<false, BLOCK, POOLS><<<grid, dim3(BLOCK), 0, s>>>(recs, pools, n_chunks, partials); \
@@ -1272,12 +1277,12 @@ int launch_norm(const ChunkRec* recs, const PoolPair& pools, int64_t n_chunks, i
     if (lanes >= 512) RLX_NORM_LAUNCH(512);
     else if (lanes == 256) RLX_NORM_LAUNCH(256);
     else if (lanes == 128) RLX_NORM_LAUNCH(128);
-    else if (g_tuning.norm_pack == 0) RLX_NORM_LAUNCH(64);
-    else if (g_tuning.norm_pack == 1) {
+    else if (norm_pack == 0) RLX_NORM_LAUNCH(64);
+    else if (norm_pack == 1) {
         // 512-element chunks: eight wavefronts per workgroup, one chunk each
         constexpr int PACK = 8;
         const dim3 pgrid((unsigned)((g + PACK - 1) / PACK));
-        if (g_tuning.norm_nt)
+        if (norm_nt)
             sumsq_partials_kernel<true, 64, POOLS, PACK><<<pgrid, dim3(64 * PACK), 0, s>>>(recs, pools, n_chunks, partials);
         else
             sumsq_partials_kernel<false, 64, POOLS, PACK><<<pgrid, dim3(64 * PACK), 0, s>>>(recs, pools, n_chunks, partials);
@@ -1287,12 +1292,12 @@ int launch_norm(const ChunkRec* recs, const PoolPair& pools, int64_t n_chunks, i
     do {                                                                                                         \
         const int64_t per_wg = (W) * (C);                                                                        \
         const dim3 pgrid((unsigned)((n_chunks + per_wg - 1) / per_wg));                                          \
-        if (g_tuning.norm_nt)                                                                                    \
+        if (norm_nt)                                                                                    \
             sumsq_small_chunks_kernel<true, POOLS, W, C><<<pgrid, dim3(64 * (W)), 0, s>>>(recs, pools, n_chunks, partials);  \
         else                                                                                                     \
             sumsq_small_chunks_kernel<false, POOLS, W, C><<<pgrid, dim3(64 * (W)), 0, s>>>(recs, pools, n_chunks, partials); \
     } while (0)
-        if (g_tuning.norm_pack == 3) RLX_SMALL(8, 2);
+        if (norm_pack == 3) RLX_SMALL(8, 2);
         else RLX_SMALL(8, 4);
 #undef RLX_SMALL
     }
@@ -1367,7 +1372,8 @@ int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream) {
     if (!dst || !src) return RLX_ERR_INVALID_ARG;
     if (!is_aligned(dst, 4) || !is_aligned(src, 2)) return RLX_ERR_MISALIGNED;
     hipStream_t s = (hipStream_t)stream;
-    if (g_tuning.convert_variant == 2) {
+    const int64_t variant = g_tuning.convert_variant;
+    if (variant == 2) {
         int64_t grid = (n + 255) / 256;
         if (grid > 65536) grid = 65536;
         fp16_to_fp32_kernel<<<dim3((unsigned)grid), dim3(256), 0, s>>>(dst, src, n);
@@ -1377,8 +1383,8 @@ int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream) {
     // measured on 2^28 elements (1.6 GB): 128 lanes x 4 elements 6.76 TB/s; 256 x 4, one or two rounds, 6.64 / 6.40;
     // 64 x 4 x 2 6.58; 128 x 2 4.28 (too many workgroups for the dispatcher); one element per lane, grid-stride, 3.45
     int lanes = 128, e = 4, rounds = 1;                           // variant 0
-    if (g_tuning.convert_variant == 1) e = 2;
-    else if (g_tuning.convert_variant == 3) { lanes = 256; rounds = 2; }
+    if (variant == 1) e = 2;
+    else if (variant == 3) { lanes = 256; rounds = 2; }
     const int64_t span = (int64_t)lanes * e * rounds;
     const int vec_ok = is_aligned(src, 2 * (size_t)e) && is_aligned(dst, 4 * (size_t)e);
     const int64_t n_wg = (n + span - 1) / span;
@@ -1387,8 +1393,8 @@ int rlx_fp16_to_fp32(float* dst, const uint16_t* src, int64_t n, void* stream) {
         float* d = dst + first * span;
         const uint16_t* q = src + first * span;
         const int64_t left = n - first * span;
-        if (g_tuning.convert_variant == 1) convert_tile_kernel<128, 2, 1><<<dim3((unsigned)here), dim3(128), 0, s>>>(d, q, left, vec_ok);
-        else if (g_tuning.convert_variant == 3) convert_tile_kernel<256, 4, 2><<<dim3((unsigned)here), dim3(256), 0, s>>>(d, q, left, vec_ok);
+        if (variant == 1) convert_tile_kernel<128, 2, 1><<<dim3((unsigned)here), dim3(128), 0, s>>>(d, q, left, vec_ok);
+        else if (variant == 3) convert_tile_kernel<256, 4, 2><<<dim3((unsigned)here), dim3(256), 0, s>>>(d, q, left, vec_ok);
         else convert_tile_kernel<128, 4, 1><<<dim3((unsigned)here), dim3(128), 0, s>>>(d, q, left, vec_ok);
         RLX_HIP(hipGetLastError());
     }
@@ -1715,7 +1721,10 @@ int rlx_set_tuning(const char* key, int64_t value) {
         if (value > 3) return RLX_ERR_INVALID_ARG;
         g_tuning.norm_pack = value;
     }
-    else if (!strcmp(key, "final_batch")) g_tuning.final_batch = value;
+    else if (!strcmp(key, "final_batch")) {
+        if (value != 0 && value != 8 && value != 16 && value != 32 && value != 40) return RLX_ERR_INVALID_ARG;
+        g_tuning.final_batch = value;
+    }
     else if (!strcmp(key, "convert_variant")) {
         if (value >= kNumConvertVariants) return RLX_ERR_INVALID_ARG;
         g_tuning.convert_variant = value;

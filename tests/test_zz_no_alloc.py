@@ -88,3 +88,34 @@ def test_static_norm_empty_input_and_limits(B, torch_gpu):
     assert B.grad_norm_static(g16.data_ptr(), 16, 0, 0, 1.0, result.data_ptr() + 4, 0, stream) == B.ERR_MISALIGNED
     assert B.grad_norm_static(0, 16, 0, 0, 1.0, result.data_ptr(), 0, stream) == B.ERR_INVALID_ARG
     torch.cuda.synchronize()
+
+
+def test_static_norm_recorded_into_a_graph(B, torch_gpu):
+    """What the entry point is for: recorded into a HIP graph (after one eager call on the device has looked up the
+    scratch array's address) and replayed with new gradients; every replay equals the plan's norm of those gradients."""
+    torch = torch_gpu
+    n16, n32 = 200_003, 5_001
+    g16 = torch.empty(n16, dtype=torch.float16, device="cuda:0")
+    g32 = torch.empty(n32, dtype=torch.float32, device="cuda:0")
+    result = torch.zeros(2, dtype=torch.float64, device="cuda:0")
+    B.fill_f16(g16.data_ptr(), n16, 1, 0.0, 1e-3)
+    B.fill_f32(g32.data_ptr(), n32, 2, 0.0, 1e-3)
+    assert B.grad_norm_static(g16.data_ptr(), n16, g32.data_ptr(), n32, 0.25, result.data_ptr()) == B.OK
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            s = torch.cuda.current_stream().cuda_stream
+            assert B.grad_norm_static(g16.data_ptr(), n16, g32.data_ptr(), n32, 0.25, result.data_ptr(), 0, s) == B.OK
+    torch.cuda.synchronize()
+    for k in range(4):
+        B.fill_f16(g16.data_ptr(), n16, 10 + k, 0.0, 1e-3 * (k + 1))          # eager work between the replays
+        B.fill_f32(g32.data_ptr(), n32, 20 + k, 0.0, 1e-3 * (k + 1))
+        result.fill_(-1.0)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = read_device(result.data_ptr(), 16).copy()
+        want, _ = plan_result(B, g16, n16, g32, n32, 0, 0.25, 0)
+        assert np.array_equal(got, want), k
