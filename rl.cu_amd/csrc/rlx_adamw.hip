@@ -391,6 +391,86 @@ __device__ __forceinline__ void update_tile(const ChunkRec& r, int64_t off, int6
     }
 }
 
+// R sub-tiles of E * LANES elements per workgroup with the same narrow, wave-contiguous accesses as update_tile:
+// the loads of all R sub-tiles are issued before the first is used.  Kept for comparison: on Qwen3-0.6B two
+// sub-tiles per workgroup reach 6.38 TB/s and four 6.0 (a one-wavefront workgroup with two, and a 256-lane one
+// with two, 6.18 and 6.36) against 6.76 for one: more bytes per workgroup widen the window of addresses in flight.  Tiles that are not whole, aligned FP16
+// tensors with parameters go through update_tile one sub-tile after the other.
+template <int E, int LANES, int R, int SP>
+__device__ __forceinline__ void update_tile_rounds(const ChunkRec& r, int64_t off, int64_t left, int lane, Hyper h,
+                                                   const rlx_step_params* __restrict__ dev_params,
+                                                   const NormResult* __restrict__ norm, uint32_t step_flags)
+{
+    constexpr int SUB = E * LANES;
+    typedef typename Lane<E>::H HV;
+    typedef typename Lane<E>::F FV;
+    const int valign = (r.flags >> kValignShift) & 0xF;
+    const bool fast = !(r.flags & (kF32 | RLX_TENSOR_GRAD_ONLY | RLX_TENSOR_FROZEN)) && valign >= E && left >= R * SUB;
+    if (!fast) {
+#pragma unroll
+        for (int k = 0; k < R; k++)
+            update_tile<E, LANES, SP, 0, true>(r, off + k * SUB, left - k * SUB, lane, h, dev_params, norm, step_flags);
+        return;
+    }
+    if (dev_params) {
+        h.lr = dev_params->lr; h.beta1 = dev_params->beta1; h.beta2 = dev_params->beta2; h.eps = dev_params->eps;
+        h.weight_decay = dev_params->weight_decay;
+        h.bc1_inv = 1.0f / dev_params->bias_correction1;
+        h.bc2_inv = 1.0f / dev_params->bias_correction2;
+    }
+    const bool clip = norm != nullptr;
+    const float scale = clip ? norm->scale : 1.0f;
+    const float wd = (r.flags & RLX_TENSOR_NO_DECAY) ? 0.0f : h.weight_decay;
+    const bool zero_grads = (step_flags & RLX_STEP_ZERO_GRADS) != 0;
+    const bool has_master = r.master != nullptr;
+    const int64_t i0 = off + lane * E;
+    HV gw[R], pw[R];
+    FV mw[R], vw[R], ww[R];
+#pragma unroll
+    for (int k = 0; k < R; k++) {
+        const int64_t i = i0 + k * SUB;
+        gw[k] = ldg<true>((const HV*)((const uint16_t*)r.g + i));
+        mw[k] = ldg<true>((const FV*)(r.m + i));
+        vw[k] = ldg<true>((const FV*)(r.v + i));
+        if (has_master) ww[k] = ldg<true>((const FV*)(r.master + i));
+        else pw[k] = ldg<true>((const HV*)((const uint16_t*)r.p + i));
+    }
+#pragma unroll
+    for (int k = 0; k < R; k++) {
+        const int64_t i = i0 + k * SUB;
+        float g[E], m[E], v[E], w[E];
+        unpack_h<E>(gw[k], g);
+        unpack_f<E>(mw[k], m);
+        unpack_f<E>(vw[k], v);
+        if (has_master) unpack_f<E>(ww[k], w);
+        else unpack_h<E>(pw[k], w);
+        if (clip) {
+#pragma unroll
+            for (int e = 0; e < E; e++) g[e] = clip_f16(g[e], scale);
+        }
+#pragma unroll
+        for (int e = 0; e < E; e++) adamw_elem(g[e], m[e], v[e], w[e], h, wd);
+        st_stream<SP>((FV*)(r.m + i), pack_f<E>(m));
+        st_stream<SP>((FV*)(r.v + i), pack_f<E>(v));
+        if (has_master) st_stream<SP>((FV*)(r.master + i), pack_f<E>(w));
+        st_stream<SP>((HV*)((uint16_t*)r.p + i), pack_h<E>(w));
+        if (zero_grads) st_stream<SP>((HV*)((uint16_t*)r.g + i), HV{});
+    }
+}
+
+template <int E, int BLOCK, int R, int SP>
+__global__ __launch_bounds__(BLOCK) void adamw_rounds_kernel(
+    const ChunkRec* __restrict__ recs, int64_t first_tile, int64_t n_tiles, int tiles_per_chunk_log2, Hyper h,
+    const rlx_step_params* __restrict__ dev_params, const NormResult* __restrict__ norm, uint32_t step_flags)
+{
+    constexpr int TILE = E * BLOCK * R;
+    const int64_t tile = first_tile + blockIdx.x;
+    if (tile >= n_tiles) return;
+    const ChunkRec r = recs[tile >> tiles_per_chunk_log2];
+    const int64_t off = (tile & ((1 << tiles_per_chunk_log2) - 1)) * TILE;
+    update_tile_rounds<E, BLOCK, R, SP>(r, off, (int64_t)r.count - off, threadIdx.x, h, dev_params, norm, step_flags);
+}
+
 // ---------------------------------------------------------------------------------------
 // Update kernel, the shipped form: one workgroup of BLOCK lanes per tile of E*BLOCK elements.
 // K > 1: workgroups b, b+8, ... land on the same XCD; groups of 8*K tiles are permuted so
@@ -951,7 +1031,7 @@ struct Tuning {
     std::atomic<int64_t> final_batch{0};    // loads in flight per lane in the second pass of the norm; 0 = by the number of partials
 } g_tuning;
 
-constexpr int kNumUpdateVariants = 15;
+constexpr int kNumUpdateVariants = 17;
 constexpr int kNumConvertVariants = 4;
 constexpr int64_t kMaxTilesPerLaunch = 1 << 23;   // workgroups per launch; times 256 lanes stays below 2^32
 constexpr int64_t kMaxNormGrid = 1 << 22;
@@ -1094,6 +1174,22 @@ hipError_t launch_per_chunk(const ChunkRec* recs, int64_t n_chunks, const Hyper&
     return hipSuccess;
 }
 
+template <int E, int BLOCK, int R>
+hipError_t launch_rounds(const ChunkRec* recs, int64_t n_chunks, int chunk_log2, const Hyper& h,
+                         const rlx_step_params* dev_params, const NormResult* norm, uint32_t step_flags, hipStream_t s) {
+    constexpr int TILE = E * BLOCK * R;
+    const int tpc_log2 = chunk_log2 - __builtin_ctz(TILE);
+    const int64_t n_tiles = n_chunks << tpc_log2;
+    for (int64_t first = 0; first < n_tiles; first += kMaxTilesPerLaunch) {
+        const int64_t here = n_tiles - first < kMaxTilesPerLaunch ? n_tiles - first : kMaxTilesPerLaunch;
+        adamw_rounds_kernel<E, BLOCK, R, 1><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(recs, first, n_tiles, tpc_log2, h,
+                                                                                      dev_params, norm, step_flags);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
 // The compiled forms of the update ("update_variant"), by number; 0 is what ships.
 const char* const kVariantNames[kNumUpdateVariants] = {
     "adamw_tile_kernel<2,128,1,*,1,0|1>",      // 0: 2 elements x 128 lanes, sc1 nt stores; loads at once, or two
@@ -1113,6 +1209,8 @@ const char* const kVariantNames[kNumUpdateVariants] = {
     "adamw_chunk_kernel<8,256,2,false>",       // 12: 128-bit accesses, one 256-lane workgroup walks a whole chunk
     "adamw_chunk_kernel<8,256,1,true>",        // 13: the same with the shipped kernel's non-temporal loads and sc1 nt stores
     "adamw_persistent_kernel<8,4,1,true>",     // 14: the persistent form with those
+    "adamw_rounds_kernel<2,128,2,1>",          // 15: the shipped accesses, two 256-element sub-tiles per workgroup
+    "adamw_rounds_kernel<2,128,4,1>",          // 16: four sub-tiles (chunks of 1,024 elements and more)
 };
 
 // any_master: some tensor of the launch has an FP32 master copy.  Such launches, and those that clear the
@@ -1126,6 +1224,7 @@ int launch_update(const ChunkRec* recs, const ChunkRec& single, int64_t single_n
 #define RLX_V(...) e = launch_variant<__VA_ARGS__>(recs, single, single_n, n, chunk_log2, h, dev_params, norm, step_flags, s)
     int64_t variant = g_tuning.update_variant;
     if (SINGLE && variant >= 11) variant = 0;      // the table-walking forms have no flat-tensor counterpart
+    if (variant == 16 && chunk_log2 < 10) variant = 0;   // its tile is 1,024 elements
     switch (variant) {
     default:
     case 0:
@@ -1146,6 +1245,8 @@ int launch_update(const ChunkRec* recs, const ChunkRec& single, int64_t single_n
     case 12: if constexpr (!SINGLE) e = launch_per_chunk<2, false>(recs, n, h, dev_params, norm, step_flags, s); break;
     case 13: if constexpr (!SINGLE) e = launch_per_chunk<1, true>(recs, n, h, dev_params, norm, step_flags, s); break;
     case 14: if constexpr (!SINGLE) e = launch_persistent<1, true>(recs, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 15: if constexpr (!SINGLE) e = launch_rounds<2, 128, 2>(recs, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 16: if constexpr (!SINGLE) e = launch_rounds<2, 128, 4>(recs, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
     }
 #undef RLX_V
     if (e != hipSuccess) return hip_fail(e, "update kernel launch");

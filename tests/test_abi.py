@@ -126,8 +126,8 @@ def test_tuning_keys(B):
     with pytest.raises(B.RlxError):
         B.set_tuning("convert_variant", 4)
     # every update variant has a kernel name; the default names the shipped tile shape
-    names = [B.update_variant_name(v) for v in range(15)]
-    assert all(names) and len(set(names)) == 15 and B.update_variant_name(15) == ""
+    names = [B.update_variant_name(v) for v in range(17)]
+    assert all(names) and len(set(names)) == 17 and B.update_variant_name(17) == ""
     assert names[0].startswith("adamw_tile_kernel<2,128,1,") and B.update_variant_name() == names[0]
     assert "persistent" in names[11] and "chunk" in names[12]
 

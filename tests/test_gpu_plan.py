@@ -299,7 +299,8 @@ def test_every_tile_shape_and_chunk_size_gives_the_same_bits(L, host, B, torch_g
     try:
         for variant, chunk in [(0, 8192), (1, 8192), (2, 2048), (3, 512), (4, 512), (5, 65536), (6, 1024),
                                (7, 2048), (8, 8192), (9, 4096), (10, 512), (10, 8192), (11, 512), (11, 2048),
-                               (11, 65536), (12, 512), (12, 8192), (13, 2048), (14, 8192)]:
+                               (11, 65536), (12, 512), (12, 8192), (13, 2048), (14, 8192), (15, 512), (15, 8192),
+                               (16, 512), (16, 1024), (16, 8192)]:
             B.set_tuning("update_variant", variant)
             st = host.ParamStore(specs, master=master)
             st.fill("p", 1, 0.0, 0.02)
