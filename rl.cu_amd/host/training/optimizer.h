@@ -249,6 +249,8 @@ public:
     // the bias corrections formed here with powf, as in step().  step_scheduled launches the update with the
     // current entry; the device then moves on to the next entry by itself, so a captured step_scheduled can be
     // replayed with nothing written by the host in between (advance get_step() with note_replayed_steps).
+    // The table belongs to the plan: if the gradient pools move or set_embed_frozen changes, the plan is rebuilt
+    // and the schedule has to be uploaded again.
     template <class Grads>
     void upload_schedule(Grads* grads, const float* lrs, int n, hipStream_t stream = 0) {
         std::vector<rlx_step_params> steps((size_t)n);
