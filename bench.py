@@ -98,6 +98,12 @@ def cpu_baseline(O, host, sample, g_clip, hyper, step, seconds=5.0):
     n1 = min(p.size, 4 * 1024 * 1024)                                # one thread, first 4 Mi parameters
     out["single_thread"], _, _ = rate(tuple(a[:n1].copy() for a in (p, g, m, v)), 0.0, 1, 2.0)
     out["single_thread_value"] = out["single_thread"]
+    # the reference's own CPU-runnable case: one flat tensor of 1,048,576 parameters, full size (first Mi of the sample)
+    n0 = 1 << 20
+    flat = tuple(a[:n0].copy() for a in (p, g, m, v))
+    r1, _, _ = rate(flat, 0.0, 1, 1.0)
+    r16, _, _ = rate(flat, 0.0, t16, 1.0)
+    out["flat_1m"] = {"params": n0, "ms_per_step_one_thread": n0 / r1 * 1e3, "ms_per_step_%d_threads" % t16: n0 / r16 * 1e3}
     out["sample"] = ("%d-parameter slice of embed_tokens of the Qwen3-0.6B list (p, m, v after 99 steps; g of step 100 "
                      "for the update leg, g~N(0,5e-3) with max_norm 1.0 for the norm+clip+update leg); %d and %d "
                      "repeated steps in %.1f and %.1f s; oracle's threaded AdamW loop, gcc -O3, no FMA contraction, "
