@@ -1,3 +1,5 @@
+// Helpers around the optimizer for C++ callers without the reference's Trainer class.  (The header has a name of
+// its own: the reference keeps its include/training/trainer.h, which this one must not shadow on the include path.)
 // The optimizer end of Trainer::training_step for C++ callers (include/training/trainer.h:269-288
 // and :323-352; GRPO_trainer.h:508-514 calls the same two functions): optional zeroing of the
 // embedding gradients, gradient clipping by global L2 norm, one optimizer step.
@@ -79,14 +81,6 @@ private:
     OptimStepConfig config_;
     float last_grad_norm_ = 0.0f;
 };
-
-// Body for the reference's Trainer::clip_grad_norm_(Qwen3Gradients* grads, float max_norm) (trainer.h:323-352),
-// whose call sites (trainer.h:282, GRPO_trainer.h:511) then stay as they are:
-//     float clip_grad_norm_(Qwen3Gradients* grads, float max_norm) { return ::clip_grad_norm_(optimizer_, grads, max_norm); }
-template <class Grads>
-inline float clip_grad_norm_(AdamWOptimizer& optimizer, Grads* grads, float max_norm) {
-    return optimizer.clip_grad_norm_(grads, max_norm);
-}
 
 // The optimizer end of Trainer::train (include/training/trainer.h:183-225): per step set the scheduled
 // rate, obtain gradients (produce_grads(step) stands for the forward/backward passes and returns the

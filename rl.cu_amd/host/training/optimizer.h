@@ -541,3 +541,11 @@ private:
         o.fp16_master_ = o.fp16_m_ = o.fp16_v_ = o.fp32_m_ = o.fp32_v_ = nullptr;
     }
 };
+
+// Body for the reference's Trainer::clip_grad_norm_(Qwen3Gradients* grads, float max_norm) (trainer.h:323-352),
+// whose call sites (trainer.h:282, GRPO_trainer.h:511) then stay as they are:
+//     float clip_grad_norm_(Qwen3Gradients* grads, float max_norm) { return ::clip_grad_norm_(optimizer_, grads, max_norm); }
+template <class Grads>
+inline float clip_grad_norm_(AdamWOptimizer& optimizer, Grads* grads, float max_norm) {
+    return optimizer.clip_grad_norm_(grads, max_norm);
+}

@@ -15,7 +15,7 @@
 #include <string>
 #include <vector>
 
-#include "training/trainer.h"
+#include "training/optimizer.h"
 
 namespace {
 

@@ -20,7 +20,7 @@
 #include <string>
 #include <vector>
 
-#include "training/trainer.h"
+#include "training/optim_step.h"
 
 extern "C" {
 float orc_h2f(uint16_t h);

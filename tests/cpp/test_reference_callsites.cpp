@@ -19,7 +19,7 @@
 #include <string>
 #include <vector>
 
-#include "training/trainer.h"
+#include "training/optimizer.h"
 
 extern "C" {
 float orc_h2f(uint16_t h);
