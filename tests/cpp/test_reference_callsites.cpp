@@ -23,6 +23,9 @@
 
 extern "C" {
 float orc_h2f(uint16_t h);
+void orc_adamw_fp16(float*, uint16_t*, const uint16_t*, float*, float*, int64_t, float, float, float, float, float,
+                    float, float);
+void orc_adamw_fp32(float*, const float*, float*, float*, int64_t, float, float, float, float, float, float, float);
 void orc_scale_half(uint16_t*, float, int64_t);
 void orc_scale_float(float*, float, int64_t);
 float orc_clip_scale(float sum_sq, float max_norm, float* norm_out);
@@ -185,7 +188,8 @@ struct World {
     std::vector<float> w32, master, m16, v16, m32, v32;
     int step = 0;
 
-    World() {
+    explicit World(const Qwen3Config& config = Qwen3Config()) {
+        model.config = config;
         Qwen3Config& c = model.config;
         c.compute_derived();
         const size_t H = c.hidden_size;
@@ -423,6 +427,72 @@ static void test_reference_test_calls() {
     if (ok) PASS(name); else FAIL(name, "accessor or step mismatch");
 }
 
+// 7. The reference's own dimensions (Qwen3-0.6B, include/model/config.h:6-12: 595,984,384 FP16 and 65,536 FP32
+//    parameters, 7.15 GB of optimizer state): the trainer tail unchanged, two steps; the norm against the FP64 sum
+//    over all gradients, and windows of every pool (its start, both sides of the boundary between the projections,
+//    which decay, and the embedding, which does not, its end, and the whole FP32 pool) against the oracle.
+static void test_full_size_model() {
+    const char* name = "Qwen3-0.6B dimensions through the reference's call sites, windows vs oracle";
+    Qwen3Config q;
+    q.vocab_size = 151936; q.hidden_size = 1024; q.intermediate_size = 3072; q.num_hidden_layers = 28;
+    q.num_attention_heads = 16; q.num_key_value_heads = 8; q.head_dim = 128;
+    World w(q);
+    TrainingConfig cfg;
+    cfg.base_lr = 1e-4f;
+    Trainer t(cfg, &w.model, &w.grads);
+    bool ok = w.n16 == 595984384u && w.n32 == 65536u && w.proj_n == 440401920u &&
+              t.optimizer().num_fp16_params() == w.n16;
+    struct Win { size_t lo, n; };
+    const Win wins[] = {{0, 40000}, {w.proj_n - 30000, 60000}, {w.n16 - 50000, 50000}, {123456789, 33333}};
+    size_t diffs = 0;
+    bool norms = true;
+    for (int s = 0; s < 2; s++) {
+        w.new_gradients(4000 + 10 * s, 5e-3f);
+        const std::vector<uint16_t> g16 = d2h<uint16_t>(w.grads.half_pool, w.n16);
+        std::vector<float> g32 = d2h<float>(w.grads.float_pool, w.n32 + w.tail);
+        const double exact = sqrt(orc_sum_sq_half(g16.data(), (int64_t)w.n16) +
+                                  orc_sum_sq_float(g32.data(), (int64_t)(w.n32 + w.tail)));
+        t.training_step_tail(1.0f, 1);
+        HIP_CHECK(hipDeviceSynchronize());
+        const float norm = t.last_grad_norm();
+        norms = norms && fabs((double)norm - exact) <= 1e-5 * exact && norm > cfg.max_grad_norm;
+        const float scale = cfg.max_grad_norm / (norm + 1e-6f);                   // trainer.h:344
+        w.step++;
+        const float bc1 = 1.0f - powf(cfg.beta1, (float)w.step), bc2 = 1.0f - powf(cfg.beta2, (float)w.step);
+        for (const Win& win : wins) {
+            // the window's state on the host mirror (weights, master, moments), advanced by the oracle
+            std::vector<uint16_t> gw(g16.begin() + win.lo, g16.begin() + win.lo + win.n);
+            orc_scale_half(gw.data(), scale, (int64_t)win.n);
+            // elements below proj_n decay, the others do not (optimizer.h:124-140)
+            const size_t split = win.lo >= w.proj_n ? 0 : (win.lo + win.n <= w.proj_n ? win.n : w.proj_n - win.lo);
+            orc_adamw_fp16(w.master.data() + win.lo, w.w16.data() + win.lo, gw.data(), w.m16.data() + win.lo,
+                           w.v16.data() + win.lo, (int64_t)split, cfg.base_lr, cfg.beta1, cfg.beta2, cfg.opt_eps,
+                           cfg.weight_decay, bc1, bc2);
+            orc_adamw_fp16(w.master.data() + win.lo + split, w.w16.data() + win.lo + split, gw.data() + split,
+                           w.m16.data() + win.lo + split, w.v16.data() + win.lo + split, (int64_t)(win.n - split),
+                           cfg.base_lr, cfg.beta1, cfg.beta2, cfg.opt_eps, 0.0f, bc1, bc2);
+            const std::vector<uint16_t> dw = d2h<uint16_t>((const uint16_t*)w.model.weights.fp16_pool + win.lo, win.n);
+            const std::vector<float> dm = d2h<float>(t.optimizer().fp16_m() + win.lo, win.n);
+            const std::vector<float> dv = d2h<float>(t.optimizer().fp16_v() + win.lo, win.n);
+            const std::vector<float> dmas = d2h<float>(t.optimizer().fp16_master() + win.lo, win.n);
+            const std::vector<uint16_t> dg = d2h<uint16_t>((const uint16_t*)w.grads.half_pool + win.lo, win.n);
+            for (size_t i = 0; i < win.n; i++)
+                diffs += dw[i] != w.w16[win.lo + i] || memcmp(&dm[i], &w.m16[win.lo + i], 4) ||
+                         memcmp(&dv[i], &w.v16[win.lo + i], 4) || memcmp(&dmas[i], &w.master[win.lo + i], 4) ||
+                         dg[i] != gw[i];
+        }
+        orc_scale_float(g32.data(), scale, (int64_t)(w.n32 + w.tail));
+        orc_adamw_fp32(w.w32.data(), g32.data(), w.m32.data(), w.v32.data(), (int64_t)w.n32, cfg.base_lr, cfg.beta1,
+                       cfg.beta2, cfg.opt_eps, 0.0f, bc1, bc2);
+        diffs += count_diff(d2h<float>(w.model.weights.fp32_pool, w.n32), w.w32);
+        diffs += count_diff(d2h<float>(t.optimizer().fp32_v(), w.n32), w.v32);
+        diffs += count_diff(d2h<float>(w.grads.float_pool, w.n32 + w.tail), g32);
+    }
+    printf("  norm=%.6f  mismatching values in the windows over 2 steps=%zu\n", t.last_grad_norm(), diffs);
+    if (ok && norms && diffs == 0 && t.optimizer().get_step() == 2) PASS(name);
+    else FAIL(name, "ok=%d norms=%d diffs=%zu", ok, norms, diffs);
+}
+
 int main() {
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
@@ -436,6 +506,7 @@ int main() {
     test_grpo_tail(true);
     test_clip_disabled();
     test_reference_test_calls();
+    test_full_size_model();
     printf("=== %s (%d failure%s) ===\n", g_fails ? "FAILED" : "ALL PASSED", g_fails, g_fails == 1 ? "" : "s");
     return g_fails;
 }
