@@ -146,9 +146,13 @@ int64_t rlx_plan_chunk_elems(const rlx_plan* plan);
 /*
  * Global gradient L2 norm and clip scale, entirely on the device:
  * replaces the reduce half of Trainer::clip_grad_norm_ (include/training/trainer.h:323-345,
- * sum_sq_half_kernel / sum_sq_float_kernel :103-133).  Two passes without atomics:
- * one FP64 partial per chunk in table order, then one block that adds the partials in
- * a fixed order, so that the result is the same bits on every run.  Writes
+ * sum_sq_half_kernel / sum_sq_float_kernel :103-133).  No value is ever added by an atomic:
+ * one FP64 partial per chunk in table order (for plans with 512-element chunks, 16 consecutive
+ * partials are then added, in order, into one group partial), then one workgroup adds these
+ * in a fixed order, so that the result is the same bits on every run.  That last sum is a
+ * second launch, or, for launches of up to 4,096 workgroups, the tail of the first one: the
+ * workgroup that finishes last (found by counting tickets, which decides who adds but not in
+ * which order) does it.  Both forms give the same bits ("norm_fused" below chooses).  Writes
  * {sum_sq, norm = sqrtf((float)sum_sq), scale} to the plan's device result, where
  * scale = max_norm / (norm + 1e-6f) iff norm > max_norm, else 1.0f (a NaN norm gives
  * 1.0f, as the reference's comparison does; max_norm = INFINITY measures without clipping).
@@ -165,14 +169,16 @@ int rlx_plan_norm_read(rlx_plan* plan, float* norm, float* scale, double* sum_sq
 
 /* Device address of the result {double sum_sq; float norm; float scale;} (16 bytes). */
 const void* rlx_plan_norm_device_ptr(const rlx_plan* plan);
-/* Device address of the per-chunk FP64 partials (rlx_plan_num_chunks values). */
+/* Device address of the per-chunk FP64 partials (rlx_plan_num_chunks values); plans with 512-element chunks
+ * keep one group partial per 16 chunks directly behind them. */
 const double* rlx_plan_partials_device_ptr(const rlx_plan* plan);
 
 /*
  * The same two-pass norm and clip rule over two flat gradient buffers (an FP16 one, then an FP32 one: the
  * shape of half_pool / float_pool) without a plan and without allocating anything.  It has no counterpart
  * in the reference; it is for callers that cannot allocate: code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc.  The per-chunk FP64 partials go to a 2 MiB array that is part of
+ * loops, harnesses that forbid hipMalloc.  The FP64 partials (and the ticket counters of the one-launch form)
+ * go to a 2.2 MiB array that is part of
  * the library's device image (every GPU the library runs on holds it until the process ends), so at most
  * 262,144 chunks fit: more returns RLX_ERR_TOO_LARGE (chunk_elems = 0 chooses the chunk as rlx_plan_create
  * would for these two tensors, which covers about 17e9 elements; otherwise a power of two >= 512).
@@ -181,7 +187,9 @@ const double* rlx_plan_partials_device_ptr(const rlx_plan* plan);
  * Either buffer may be empty (n = 0).  Calls no hipMalloc, hipFree or other allocating routine; the first call
  * on a device looks up the array's address there (make that call outside a graph capture).  All calls on one
  * GPU share the array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream
- * do not.  Nothing in the array has to start at zero: every call writes each slot that it later reads.
+ * do not.  The partials need not start at zero: every call writes each slot that it later reads.  The ticket
+ * counters must, and do: they are zero in the image and the workgroup that draws a counter's last ticket sets
+ * it back to zero, so every call that runs to its end leaves them at zero for the next.
  */
 int rlx_grad_norm_static(const uint16_t* half_grads, int64_t n_half, const float* float_grads, int64_t n_float,
                          int64_t chunk_elems, float max_norm, void* result_dev, void* stream);
@@ -228,17 +236,28 @@ int rlx_plan_adamw_dev(rlx_plan* plan, const rlx_step_params* dev_params, int st
  * the values from the host each time (optimizer.h:119-147).
  *
  * rlx_plan_schedule_upload: every entry is validated like the arguments of rlx_plan_adamw (finite, bias
- * corrections not 0: RLX_ERR_BAD_HYPER otherwise, nothing uploaded).  Waits for `stream`, allocates when the
- * table grows and copies synchronously: call it outside the step loop and outside a graph capture.  The next
- * scheduled update reads entry 0.
+ * corrections not 0: RLX_ERR_BAD_HYPER otherwise, nothing uploaded).  Waits for the whole device
+ * (hipDeviceSynchronize: scheduled updates of this plan that are still running, on `stream` or on any other
+ * stream, replays of a recorded step included, read the old table), allocates when the table grows and copies
+ * synchronously: call it outside the step loop and outside a graph capture.  `stream` is not otherwise used.
+ * The next scheduled update reads entry 0.
+ * A recorded rlx_plan_adamw_scheduled stays valid across uploads, of any length: the launch names only a small
+ * header whose device address is fixed from the first upload until rlx_plan_destroy; the table's address and
+ * length are read from that header when the kernel runs.  Record the step once, after the first upload, and
+ * replay it through every later window.
  * rlx_plan_adamw_scheduled: the update of rlx_plan_adamw_dev with the current entry, then the advance.  After
- * the last entry has been used, that entry stays current (upload the next window before that happens).
+ * the last entry has been used, that entry stays current (upload the next window before that happens);
+ * updates that run with it again are counted (rlx_plan_schedule_overrun).
  * rlx_plan_schedule_position: how many scheduled steps have run since the upload (saturating at n_steps) and
  * the table's length; waits for `stream`.  Either out pointer may be NULL.
+ * rlx_plan_schedule_overrun: how many scheduled updates since the upload ran after the table had been used up,
+ * i.e. with the last entry's learning rate and bias corrections instead of their own (0 in a correct run);
+ * waits for `stream`.
  */
 int rlx_plan_schedule_upload(rlx_plan* plan, const rlx_step_params* steps, int64_t n_steps, void* stream);
 int rlx_plan_adamw_scheduled(rlx_plan* plan, int step_flags, void* stream);
 int rlx_plan_schedule_position(rlx_plan* plan, int64_t* steps_taken, int64_t* n_steps, void* stream);
+int rlx_plan_schedule_overrun(rlx_plan* plan, int64_t* overrun, void* stream);
 
 /* ------------------------------------------------------------------------------------
  * Launch tuning (process-wide; for measurement).  Unknown keys return RLX_ERR_INVALID_ARG.
@@ -256,6 +275,9 @@ int rlx_plan_schedule_position(rlx_plan* plan, int64_t* steps_taken, int64_t* n_
  *                     wavefront), 2 = thirty-two (four per wavefront, default), 3 = sixteen
  *   "final_batch"     loads that a lane of the norm's second pass keeps in flight: 8, 16, 32, 40, or
  *                     0 = chosen from the number of partials (default)
+ *   "norm_fused"      who adds the norm's partials: 0 = always a second launch of one workgroup; 1 = the
+ *                     workgroup of the first launch that finishes last, whenever that launch has at most
+ *                     8,192 workgroups; 2 = that for launches of up to 4,096 workgroups (default).  Same bits.
  *   "convert_variant" rlx_fp16_to_fp32: 0 = 128 lanes x 4 elements per workgroup (default),
  *                     1 = 128 lanes x 2 elements, 2 = one element per lane, grid-stride,
  *                     3 = 256 lanes x 4 elements x 2 rounds

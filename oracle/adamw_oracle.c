@@ -349,8 +349,24 @@ int64_t orc_sumsq_mirror_partials(const void* g, int is_f32, int64_t n, int chun
 }
 
 /*
- * Final pass: 1024 threads, thread t adds partials t, t+1024, ... in order (FP64),
- * then a halving tree (512, 256, ..., 1) in FP64.
+ * Group partials (plans with 512-element chunks only): 16 consecutive chunk partials are
+ * added in FP64, in index order, starting from 0.0.  Returns the number of groups written.
+ */
+int64_t orc_sumsq_mirror_groups(const double* partials, int64_t n_partials, double* groups)
+{
+    int64_t k = 0;
+    for (int64_t first = 0; first < n_partials; first += 16) {
+        double total = 0.0;
+        for (int64_t i = first; i < first + 16 && i < n_partials; i++) total += partials[i];
+        groups[k++] = total;
+    }
+    return k;
+}
+
+/*
+ * Final pass: 1024 threads, thread t adds its values t, t+1024, ... in order (FP64),
+ * then a halving tree (512, 256, ..., 1) in FP64.  The values are the chunk partials, or
+ * the group partials for 512-element chunks (orc_sumsq_mirror_total picks).
  */
 double orc_sumsq_mirror_final(const double* partials, int64_t n_partials)
 {
@@ -363,6 +379,18 @@ double orc_sumsq_mirror_final(const double* partials, int64_t n_partials)
     for (int s = 512; s >= 1; s >>= 1)
         for (int t = 0; t < s; t++) acc[t] = acc[t] + acc[t + s];
     return acc[0];
+}
+
+/* The device's sum of squares from the per-chunk partials of a plan with chunks of `chunk` elements. */
+double orc_sumsq_mirror_total(const double* partials, int64_t n_partials, int chunk)
+{
+    if (chunk != 512) return orc_sumsq_mirror_final(partials, n_partials);
+    int64_t n_groups = (n_partials + 15) / 16;
+    double* groups = (double*)malloc(sizeof(double) * (size_t)(n_groups > 0 ? n_groups : 1));
+    orc_sumsq_mirror_groups(partials, n_partials, groups);
+    double total = orc_sumsq_mirror_final(groups, n_groups);
+    free(groups);
+    return total;
 }
 
 /* ------------------------------------------------------------------ */

@@ -53,6 +53,8 @@ def _load():
         "orc_clip_grad_norm": ([vp, i64, vp, i64, f, f32p], f),
         "orc_sumsq_mirror_partials": ([vp, i32, i64, i32, vp], i64),
         "orc_sumsq_mirror_final": ([vp, i64], C.c_double),
+        "orc_sumsq_mirror_groups": ([vp, i64, vp], i64),
+        "orc_sumsq_mirror_total": ([vp, i64, i32], C.c_double),
         "orc_fill_f16": ([vp, i64, u64, i64, f, f, u32, i64, u32], None),
         "orc_fill_f32": ([vp, i64, u64, i64, f, f, u32, i64, u32], None),
         "orc_step_fp16_threaded": ([vp, vp, vp, vp, vp, i64] + hyper + [f, i32], f),
@@ -158,10 +160,25 @@ def clip_grad_norm(half_pool, float_pool, max_norm):
     return float(norm), float(sc.value)
 
 
-def sumsq_mirror_final(partials):
-    """The fixed-order FP64 sum of per-chunk partials (pass 2 of the device's norm)."""
-    allp = np.ascontiguousarray(partials, dtype=np.float64)
+def sumsq_mirror_final(values):
+    """The fixed-order FP64 sum of the last step of the device's norm (over chunk partials, or over group
+    partials for 512-element chunks)."""
+    allp = np.ascontiguousarray(values, dtype=np.float64)
     return float(lib.orc_sumsq_mirror_final(_p(allp, F64), allp.size))
+
+
+def sumsq_mirror_groups(partials):
+    """Group partials of a plan with 512-element chunks: 16 consecutive chunk partials added in order."""
+    allp = np.ascontiguousarray(partials, dtype=np.float64)
+    out = np.empty(max((allp.size + 15) // 16, 1), np.float64)
+    k = lib.orc_sumsq_mirror_groups(_p(allp, F64), allp.size, _p(out, F64))
+    return out[:k]
+
+
+def sumsq_mirror_total(partials, chunk):
+    """The device's sum of squares from its per-chunk partials, for a plan with chunks of `chunk` elements."""
+    allp = np.ascontiguousarray(partials, dtype=np.float64)
+    return float(lib.orc_sumsq_mirror_total(_p(allp, F64), allp.size, chunk))
 
 
 def sumsq_mirror(grads, chunk):
@@ -176,7 +193,7 @@ def sumsq_mirror(grads, chunk):
         assert got == k
         parts.append(buf[:k])
     allp = np.ascontiguousarray(np.concatenate(parts)) if parts else np.zeros(0, np.float64)
-    return float(lib.orc_sumsq_mirror_final(_p(allp, F64), allp.size)), allp
+    return float(lib.orc_sumsq_mirror_total(_p(allp, F64), allp.size, chunk)), allp
 
 
 def fill_f16(n, seed, mean, std, first=0, flags=0, row_len=0, zero_rows_below=0):

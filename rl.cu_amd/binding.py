@@ -64,6 +64,7 @@ SIGNATURES = {
     "rlx_plan_schedule_upload": ([_VP, C.POINTER(StepParams), _I64, _VP], _INT),
     "rlx_plan_adamw_scheduled": ([_VP, _INT, _VP], _INT),
     "rlx_plan_schedule_position": ([_VP, C.POINTER(_I64), C.POINTER(_I64), _VP], _INT),
+    "rlx_plan_schedule_overrun": ([_VP, C.POINTER(_I64), _VP], _INT),
     "rlx_update_variant_name": ([_I64], C.c_char_p),
     "rlx_set_tuning": ([C.c_char_p, _I64], _INT),
     "rlx_get_tuning": ([C.c_char_p], _I64),
@@ -74,24 +75,33 @@ SIGNATURES = {
 _lib = None
 
 
-ABI_VERSION = 108        # rlx_version() of the library this binding was written against
+ABI_VERSION = 109        # rlx_version() of the library this binding was written against
 
 
 def load():
-    """Loads the built library.  If it is missing, or was built from other sources than the ones in the tree
-    (the build leaves a hash of its sources next to the library), it is compiled first; if that fails, or the
-    loaded library reports another ABI version than this binding expects, loading raises.  There is no CPU
-    fallback of any kind."""
+    """Loads the built library; there is no CPU fallback of any kind.
+    Missing library: it is compiled first, and loading raises if that fails.
+    Library whose source stamp (the hash of its sources that this package's build leaves next to it) differs from
+    the tree: it is compiled again; if that cannot be done (no hipcc on this machine) the existing library is
+    loaded with a warning.
+    Library without a stamp (built with the documented hipcc line or by CMake): loaded as it is.
+    In every case the loaded library must report the ABI version that this binding was written against."""
     global _lib
     if _lib is not None:
         return _lib
     from . import build as _build
-    if not _build.is_current():
-        why = "not built" if not os.path.exists(LIB_PATH) else "built from other sources than the tree holds"
+    if not os.path.exists(LIB_PATH):
         try:
             _build.build_library()
         except Exception as exc:
-            raise RuntimeError("librlx_adamw.so is %s (%s) and building it failed: %s" % (why, LIB_PATH, exc))
+            raise RuntimeError("librlx_adamw.so is not built (%s) and building it failed: %s" % (LIB_PATH, exc))
+    elif _build.is_stale():
+        try:
+            _build.build_library()
+        except Exception as exc:
+            import warnings
+            warnings.warn("librlx_adamw.so was built from other sources than the tree holds and could not be rebuilt "
+                          "(%s); loading it as it is" % exc)
     try:
         # torch, when present, brings its own HIP runtime: load it first so that this library
         # binds to the same runtime instance as the tensors it is handed.
@@ -252,6 +262,12 @@ class Plan:
         check(load().rlx_plan_schedule_position(self._h, C.byref(taken), C.byref(total), stream),
               "rlx_plan_schedule_position")
         return taken.value, total.value
+
+    def schedule_overrun(self, stream=0):
+        """Blocking.  Scheduled updates since the upload that ran after the table had been used up."""
+        over = _I64()
+        check(load().rlx_plan_schedule_overrun(self._h, C.byref(over), stream), "rlx_plan_schedule_overrun")
+        return over.value
 
     def destroy(self):
         if self._h is not None:

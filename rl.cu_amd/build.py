@@ -41,6 +41,15 @@ def is_current():
         return False
 
 
+def is_stale():
+    """True if the library carries a source stamp and the stamp differs from the sources in the tree.  A library
+    without a stamp was built by other means (the documented hipcc line, CMake) and is not judged here."""
+    try:
+        return os.path.exists(OUT) and os.path.exists(STAMP) and open(STAMP).read().strip() != source_hash()
+    except OSError:
+        return False
+
+
 def hipcc_path():
     for cand in (shutil.which("hipcc"), "/opt/rocm/bin/hipcc"):
         if cand and os.path.exists(cand):

@@ -40,12 +40,16 @@
 
 #include "rlx_adamw.h"
 
-// Per-chunk FP64 partials of rlx_grad_norm_static, the entry point for callers that cannot allocate: part of
-// the library's device image (2 MiB on every GPU the library runs on, until the process ends).  The name
-// stands for the array only in device code; host code uses the address that hipGetSymbolAddress returns for
-// the current device (static_scratch below), never the name.
+// Intermediate sums of rlx_grad_norm_static, the entry point for callers that cannot allocate: part of the
+// library's device image (2.2 MiB on every GPU the library runs on, until the process ends).  Layout, in
+// doubles: [0, 2^18) per-chunk FP64 partials; [2^18, 2^18 + 2^14) group partials (one per 16 chunks, used with
+// 512-element chunks); then 16.5 KiB of 32-bit ticket counters, which start at zero in the image and which every
+// launch leaves at zero again.  The name stands for the array only in device code; host code uses the address
+// that hipGetSymbolAddress returns for the current device (static_scratch below), never the name.
 constexpr int64_t kStaticMaxPartials = 1 << 18;
-static __device__ __align__(256) double scratch[kStaticMaxPartials];
+constexpr int64_t kStaticMaxGroups = kStaticMaxPartials / 16;
+constexpr int64_t kStaticTicketDoubles = (8192 / 64 + 1) * 32 / 2;      // kTicketWords 32-bit words
+static __device__ __align__(256) double scratch[kStaticMaxPartials + kStaticMaxGroups + kStaticTicketDoubles];
 
 namespace {
 
@@ -71,13 +75,15 @@ struct ChunkRec {
     float* v;
     float* master;
     uint32_t count;      // elements in this chunk (the last chunk of a tensor may be short)
-    uint32_t flags;      // RLX_TENSOR_* | kF32 | valign << kValignShift
+    uint32_t flags;      // RLX_TENSOR_* | kF32 | valign << kValignShift | galign << kGalignShift
     int64_t pad[2];
 };
 static_assert(sizeof(ChunkRec) == 64, "ChunkRec is one 64-byte record");
 constexpr uint32_t kF32 = 0x10;               // FP32 parameter and gradient
 constexpr int kValignShift = 8;               // flags bits 8..11: widest lane vector (1,2,4,8 elements)
                                               // for which every stream of the chunk is aligned
+constexpr int kGalignShift = 12;              // flags bits 12..15: the same for the gradient stream alone (the
+                                              // norm and the scale pass touch nothing else)
 
 struct NormResult {
     double sum_sq;
@@ -88,6 +94,19 @@ struct NormResult {
 struct Hyper {
     float lr, beta1, beta2, eps, weight_decay, bc1_inv, bc2_inv;
 };
+
+// Device-resident state of a plan's step table (host-free replay).  One allocation whose address stays the same
+// from the first upload until the plan is destroyed: recorded launches name it and nothing else.
+struct SchedHeader {
+    rlx_step_params current;         // the entry that the next scheduled update reads (first member: the update
+                                     // kernel is handed the header's address as its hyper-parameters)
+    uint32_t pad0;
+    int64_t taken;                   // scheduled steps since the upload, saturating at len
+    const rlx_step_params* table;    // the uploaded entries
+    int64_t len;
+    int64_t overrun;                 // scheduled updates that ran after the table had been used up
+};
+static_assert(sizeof(SchedHeader) == 64 && sizeof(rlx_step_params) == 28, "one 64-byte header");
 
 // Two flat gradient buffers described by value (an FP16 one followed by an FP32 one, the shape of
 // the reference's half_pool / float_pool): the chunks that a plan over these two tensors would
@@ -273,9 +292,11 @@ __device__ __forceinline__ void update_scalar32(const ChunkRec& r, int64_t i, co
 // SP: 1 = system-scope non-temporal stores, 0 = non-temporal stores, 2 = ordinary stores; NTL: non-temporal loads.
 // PH: 0 = a lane issues the tile's four loads at once; 1 = tiles that write four streams (master copy,
 // gradient clearing) issue their loads, and with a master copy their stores, two at a time.
+// CLIP: the gradients are multiplied by the clip scale at `norm` first (a compile-time choice, so that the
+// plain and the fused-clip update are two kernels with two names in a profile).
 // ---------------------------------------------------------------------------------------
 
-template <int E, int LANES, int SP, int PH, bool NTL = true>
+template <int E, int LANES, int SP, int PH, bool NTL, bool CLIP>
 __device__ __forceinline__ void update_tile(const ChunkRec& r, int64_t off, int64_t left, int lane, Hyper h,
                                             const rlx_step_params* __restrict__ dev_params,
                                             const NormResult* __restrict__ norm, uint32_t step_flags)
@@ -314,8 +335,9 @@ __device__ __forceinline__ void update_tile(const ChunkRec& r, int64_t off, int6
         h.bc1_inv = 1.0f / dev_params->bias_correction1;
         h.bc2_inv = 1.0f / dev_params->bias_correction2;
     }
-    const bool clip = norm != nullptr;
-    const float scale = clip ? norm->scale : 1.0f;
+    constexpr bool clip = CLIP;
+    float scale = 1.0f;
+    if constexpr (CLIP) scale = norm->scale;
     const float wd = (r.flags & RLX_TENSOR_NO_DECAY) ? 0.0f : h.weight_decay;
 
     if (!vec) {
@@ -396,7 +418,7 @@ __device__ __forceinline__ void update_tile(const ChunkRec& r, int64_t off, int6
 // sub-tiles per workgroup reach 6.38 TB/s and four 6.0 (a one-wavefront workgroup with two, and a 256-lane one
 // with two, 6.18 and 6.36) against 6.76 for one: more bytes per workgroup widen the window of addresses in flight.  Tiles that are not whole, aligned FP16
 // tensors with parameters go through update_tile one sub-tile after the other.
-template <int E, int LANES, int R, int SP>
+template <int E, int LANES, int R, int SP, bool CLIP>
 __device__ __forceinline__ void update_tile_rounds(const ChunkRec& r, int64_t off, int64_t left, int lane, Hyper h,
                                                    const rlx_step_params* __restrict__ dev_params,
                                                    const NormResult* __restrict__ norm, uint32_t step_flags)
@@ -409,7 +431,7 @@ __device__ __forceinline__ void update_tile_rounds(const ChunkRec& r, int64_t of
     if (!fast) {
 #pragma unroll
         for (int k = 0; k < R; k++)
-            update_tile<E, LANES, SP, 0, true>(r, off + k * SUB, left - k * SUB, lane, h, dev_params, norm, step_flags);
+            update_tile<E, LANES, SP, 0, true, CLIP>(r, off + k * SUB, left - k * SUB, lane, h, dev_params, norm, step_flags);
         return;
     }
     if (dev_params) {
@@ -418,8 +440,9 @@ __device__ __forceinline__ void update_tile_rounds(const ChunkRec& r, int64_t of
         h.bc1_inv = 1.0f / dev_params->bias_correction1;
         h.bc2_inv = 1.0f / dev_params->bias_correction2;
     }
-    const bool clip = norm != nullptr;
-    const float scale = clip ? norm->scale : 1.0f;
+    constexpr bool clip = CLIP;
+    float scale = 1.0f;
+    if constexpr (CLIP) scale = norm->scale;
     const float wd = (r.flags & RLX_TENSOR_NO_DECAY) ? 0.0f : h.weight_decay;
     const bool zero_grads = (step_flags & RLX_STEP_ZERO_GRADS) != 0;
     const bool has_master = r.master != nullptr;
@@ -458,7 +481,7 @@ __device__ __forceinline__ void update_tile_rounds(const ChunkRec& r, int64_t of
     }
 }
 
-template <int E, int BLOCK, int R, int SP>
+template <int E, int BLOCK, int R, int SP, bool CLIP>
 __global__ __launch_bounds__(BLOCK) void adamw_rounds_kernel(
     const ChunkRec* __restrict__ recs, int64_t first_tile, int64_t n_tiles, int tiles_per_chunk_log2, Hyper h,
     const rlx_step_params* __restrict__ dev_params, const NormResult* __restrict__ norm, uint32_t step_flags)
@@ -468,7 +491,7 @@ __global__ __launch_bounds__(BLOCK) void adamw_rounds_kernel(
     if (tile >= n_tiles) return;
     const ChunkRec r = recs[tile >> tiles_per_chunk_log2];
     const int64_t off = (tile & ((1 << tiles_per_chunk_log2) - 1)) * TILE;
-    update_tile_rounds<E, BLOCK, R, SP>(r, off, (int64_t)r.count - off, threadIdx.x, h, dev_params, norm, step_flags);
+    update_tile_rounds<E, BLOCK, R, SP, CLIP>(r, off, (int64_t)r.count - off, threadIdx.x, h, dev_params, norm, step_flags);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -478,7 +501,7 @@ __global__ __launch_bounds__(BLOCK) void adamw_rounds_kernel(
 // SINGLE: one flat tensor passed by value (the operator API); otherwise the plan's records.
 // ---------------------------------------------------------------------------------------
 
-template <int E, int BLOCK, int K, bool SINGLE, int SP, int PH, bool NTL>
+template <int E, int BLOCK, int K, bool SINGLE, int SP, int PH, bool NTL, bool CLIP>
 __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
     const ChunkRec* __restrict__ recs, ChunkRec single, int64_t single_n, int64_t first_tile, int64_t n_tiles,
     int tiles_per_chunk_log2, Hyper h, const rlx_step_params* __restrict__ dev_params,
@@ -505,7 +528,7 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         off = (tile & ((1 << tiles_per_chunk_log2) - 1)) * TILE;
         left = (int64_t)r.count - off;
     }
-    update_tile<E, BLOCK, SP, PH, NTL>(r, off, left, threadIdx.x, h, dev_params, norm, step_flags);
+    update_tile<E, BLOCK, SP, PH, NTL, CLIP>(r, off, left, threadIdx.x, h, dev_params, norm, step_flags);
 }
 
 // ---------------------------------------------------------------------------------------
@@ -517,7 +540,7 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
 // adamw_chunk_kernel: one workgroup per chunk that walks its chunk in groups of E*BLOCK elements.
 // ---------------------------------------------------------------------------------------
 
-template <int E, int WAVES, int SP, bool NTL>
+template <int E, int WAVES, int SP, bool NTL, bool CLIP>
 __global__ __launch_bounds__(64 * WAVES) void adamw_persistent_kernel(
     const ChunkRec* __restrict__ recs, int64_t n_tiles, int tiles_per_chunk_log2, Hyper h,
     const rlx_step_params* __restrict__ dev_params, const NormResult* __restrict__ norm, uint32_t step_flags)
@@ -527,11 +550,11 @@ __global__ __launch_bounds__(64 * WAVES) void adamw_persistent_kernel(
     for (int64_t tile = (int64_t)blockIdx.x * WAVES + wave; tile < n_tiles; tile += (int64_t)gridDim.x * WAVES) {
         const ChunkRec r = recs[tile >> tiles_per_chunk_log2];
         const int64_t off = (tile & ((1 << tiles_per_chunk_log2) - 1)) * TILE;
-        update_tile<E, 64, SP, 0, NTL>(r, off, (int64_t)r.count - off, lane, h, dev_params, norm, step_flags);
+        update_tile<E, 64, SP, 0, NTL, CLIP>(r, off, (int64_t)r.count - off, lane, h, dev_params, norm, step_flags);
     }
 }
 
-template <int E, int BLOCK, int SP, bool NTL>
+template <int E, int BLOCK, int SP, bool NTL, bool CLIP>
 __global__ __launch_bounds__(BLOCK) void adamw_chunk_kernel(
     const ChunkRec* __restrict__ recs, int64_t first_chunk, int64_t n_chunks, Hyper h,
     const rlx_step_params* __restrict__ dev_params, const NormResult* __restrict__ norm, uint32_t step_flags)
@@ -541,18 +564,125 @@ __global__ __launch_bounds__(BLOCK) void adamw_chunk_kernel(
     if (c >= n_chunks) return;
     const ChunkRec r = recs[c];
     for (int64_t off = 0; off < (int64_t)r.count; off += TILE)
-        update_tile<E, BLOCK, SP, 0, NTL>(r, off, (int64_t)r.count - off, threadIdx.x, h, dev_params, norm, step_flags);
+        update_tile<E, BLOCK, SP, 0, NTL, CLIP>(r, off, (int64_t)r.count - off, threadIdx.x, h, dev_params, norm, step_flags);
 }
 
 // ---------------------------------------------------------------------------------------
-// Norm pass 1: one workgroup per chunk, one FP64 partial per chunk in the chunk's own slot.
-// BLOCK = min(512, chunk_elems / 8) lanes, so that small chunks do not launch idle wavefronts.
-// Order inside a chunk (restated on the CPU by the test oracle): lane t of BLOCK adds x*x of its
-// 8-element groups t, t+BLOCK, ... element by element into one FP32 accumulator; the 64
-// lanes of a wavefront combine by xor butterfly with masks 32,16,8,4,2,1; the BLOCK/64
-// wavefront sums go through LDS and are added in FP64 in wavefront order.  (512 lanes with
-// two 128-bit reads each measured 7.3 TB/s as a stand-alone stream, 256 lanes with four 6.95.)
+// The norm.  Order of the sum (restated on the CPU by the test oracle), a pure function of the data and the plan:
+//   1. per chunk: lane t of BLOCK = min(512, chunk_elems / 8) adds x*x of its 8-element groups t, t+BLOCK, ...
+//      element by element into one FP32 accumulator; the 64 lanes of a wavefront combine by xor butterfly with
+//      masks 32,16,8,4,2,1; the BLOCK/64 wavefront sums are added in FP64 in wavefront order: one FP64 partial
+//      per chunk in the chunk's own slot;
+//   2. plans with 512-element chunks (lists of thousands of small tensors) only: 16 consecutive chunk partials
+//      are added in FP64, in index order, into one group partial (so that the last step reads a sixteenth);
+//   3. the values of step 2 (of step 1 for larger chunks) are added in FP64 by 1,024 (virtual) threads, thread t
+//      taking t, t+1024, ... in order, then by a halving tree.
+// Steps 1-2 are one launch.  Step 3 is either a second launch of one workgroup, or the tail of the first launch:
+// every workgroup takes a ticket when its partials are written, and the workgroup that draws the last ticket
+// adds them up.  The tickets decide who adds, never in which order, so both forms give the same bits; no
+// workgroup ever waits for another.
 // ---------------------------------------------------------------------------------------
+
+constexpr int kGroupChunks = 16;              // 512-element chunks per group partial
+constexpr int kTicketGroup = 64;              // workgroups per first-level ticket counter
+constexpr int kTicketStride = 32;             // 32-bit words from one counter to the next (128 bytes: a line each)
+constexpr int64_t kMaxFusedWgs = 8192;        // largest grid whose last workgroup adds the partials itself
+constexpr int64_t kTicketWords = (kMaxFusedWgs / kTicketGroup + 1) * kTicketStride;
+static_assert(kStaticTicketDoubles * 2 == kTicketWords && kStaticMaxGroups * kGroupChunks == kStaticMaxPartials,
+              "the static scratch holds the partials, their groups and the tickets of the largest call");
+
+// What the workgroup that finishes last needs for step 3.
+struct NormTail {
+    const double* values;        // per-chunk partials, or per-group partials for 512-element chunks
+    int64_t n_values;
+    float max_norm;
+    NormResult* out;
+    uint32_t* tickets;           // [0]: second-level counter; [(1 + g) * kTicketStride]: counter of workgroups
+                                 // 64g .. 64g+63.  All zero between launches.
+};
+
+// The sum, the norm and the clip scale (trainer.h:341-345: strict '>' and +1e-6f in the denominator).
+__device__ __forceinline__ void write_norm_result(double sum_sq, float max_norm, NormResult* __restrict__ out) {
+    const float norm = __builtin_sqrtf((float)sum_sq);
+    float scale = 1.0f;
+    if (norm > max_norm) scale = max_norm / (norm + 1e-6f);
+    out->sum_sq = sum_sq;
+    out->norm = norm;
+    out->scale = scale;
+}
+
+// Step 3 by a workgroup of NTHREADS lanes: lane `tid` runs the virtual threads tid, tid + NTHREADS, ... of 1,024,
+// each with an accumulator of its own, so the result does not depend on NTHREADS.  ROUNDS rounds of 1,024 values
+// are requested before the first is added (in index order: the same sum as one at a time).  Slots beyond the end
+// read as +0.0, which leaves a sum of squares (never negative zero) unchanged bit for bit.  COHERENT: the values
+// were written by other workgroups of the same launch; they are read with device-scope loads.
+// `lds`: 1,024 doubles.  Returns the total in every lane.
+template <int NTHREADS, int ROUNDS, bool COHERENT>
+__device__ __forceinline__ double fixed_order_sum(const double* vals, int64_t n, double* lds, int tid) {
+    constexpr int V = kFinalBlock / NTHREADS;
+    double a[V];
+#pragma unroll
+    for (int v = 0; v < V; v++) a[v] = 0.0;
+    for (int64_t base = 0; base < n; base += (int64_t)ROUNDS * kFinalBlock) {
+        double x[ROUNDS][V];
+#pragma unroll
+        for (int b = 0; b < ROUNDS; b++) {
+#pragma unroll
+            for (int v = 0; v < V; v++) {
+                const int64_t j = base + (int64_t)b * kFinalBlock + v * NTHREADS + tid;
+                double y = 0.0;
+                if (j < n) {
+                    if constexpr (COHERENT) y = __hip_atomic_load(vals + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    else y = vals[j];
+                }
+                x[b][v] = y;
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < ROUNDS; b++) {
+#pragma unroll
+            for (int v = 0; v < V; v++) a[v] += x[b][v];
+        }
+    }
+#pragma unroll
+    for (int v = 0; v < V; v++) lds[v * NTHREADS + tid] = a[v];
+    __syncthreads();
+    for (int s = kFinalBlock / 2; s >= 1; s >>= 1) {
+        for (int i = tid; i < s; i += NTHREADS) lds[i] = lds[i] + lds[i + s];
+        __syncthreads();
+    }
+    return lds[0];
+}
+
+// True in every lane of exactly one workgroup of the launch: the one that takes its ticket last.  Everything the
+// final sum reads must have been stored by lanes of the workgroup's first wavefront before the call.  Two levels
+// of counters (64 workgroups share a first-level counter, the last of each 64 takes a second-level ticket), so
+// that thousands of workgroups finishing together do not queue on one address.  Whoever draws a counter's last
+// ticket puts the counter back to zero for the next launch.
+__device__ __forceinline__ bool last_workgroup(uint32_t* tickets, int* lds_flag) {
+    if (threadIdx.x < 64) {
+        __threadfence();                    // this wavefront's partials are visible device-wide before its ticket
+        if (threadIdx.x == 0) {
+            const uint32_t n_wg = gridDim.x, grp = blockIdx.x / kTicketGroup;
+            const uint32_t n_grp = (n_wg + kTicketGroup - 1) / kTicketGroup;
+            const uint32_t in_grp = grp + 1 < n_grp ? (uint32_t)kTicketGroup : n_wg - grp * kTicketGroup;
+            uint32_t* c1 = tickets + (size_t)(1 + grp) * kTicketStride;
+            int last = 0;
+            if (__hip_atomic_fetch_add(c1, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == in_grp - 1) {
+                __hip_atomic_store(c1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                if (__hip_atomic_fetch_add(tickets, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == n_grp - 1) {
+                    __hip_atomic_store(tickets, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                    last = 1;
+                }
+            }
+            *lds_flag = last;
+        }
+    }
+    __syncthreads();
+    const bool last = *lds_flag != 0;
+    if (last) __threadfence();              // what the other workgroups released is visible to this one's loads
+    return last;
+}
 
 // Chunk c of a PoolPair as the record that a plan would hold for it (only the fields the norm reads).
 __device__ __forceinline__ ChunkRec pool_chunk(const PoolPair& pp, int64_t c) {
@@ -572,17 +702,109 @@ __device__ __forceinline__ ChunkRec pool_chunk(const PoolPair& pp, int64_t c) {
     return r;
 }
 
+// Sum of squares of this lane's share of one chunk: lane `tid` of BLOCK adds its 8-element groups tid,
+// tid + BLOCK, ... element by element into one FP32 accumulator.
+template <bool NT, int BLOCK>
+__device__ __forceinline__ float chunk_lane_sumsq(const ChunkRec& r, int tid) {
+    constexpr int kNormGroup = BLOCK * kVec;
+    const int64_t count = r.count;
+    const bool aligned = ((r.flags >> kGalignShift) & 0xF) >= 8;
+    float acc = 0.0f;
+    if (r.flags & RLX_TENSOR_FROZEN) {
+        // gradients of a frozen tensor count as zero (the reference clears them before the norm)
+    } else if (!(r.flags & kF32)) {
+        const uint16_t* g = (const uint16_t*)r.g;
+        int64_t done = 0;
+        if (aligned) {
+            for (; done + 2 * (int64_t)kNormGroup <= count; done += 2 * (int64_t)kNormGroup) {
+                u32x4 x[2];
+#pragma unroll
+                for (int j = 0; j < 2; j++)
+                    x[j] = ldg<NT>((const u32x4*)(g + done + (int64_t)(j * BLOCK + tid) * kVec));
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        float a = h2f(x[j][k] & 0xFFFFu), b = h2f(x[j][k] >> 16);
+                        acc = acc + a * a;
+                        acc = acc + b * b;
+                    }
+                }
+            }
+        }
+        for (; done < count; done += kNormGroup) {
+            const int64_t off = done + (int64_t)tid * kVec;
+            if (aligned && off + kVec <= count) {
+                u32x4 x = ldg<NT>((const u32x4*)(g + off));
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    float a = h2f(x[k] & 0xFFFFu), b = h2f(x[k] >> 16);
+                    acc = acc + a * a;
+                    acc = acc + b * b;
+                }
+            } else if (aligned && off < count) {
+                // the tensor's last, partial group: its 16-byte granule starts inside the tensor, so one
+                // aligned load cannot leave the tensor's last page; what lies beyond the end is read but
+                // counts as zero (acc + 0 leaves a sum of squares as it is).  Element by element this
+                // lane would wait for up to seven loads one after another, and its workgroup with it.
+                u32x4 x = ldg<NT>((const u32x4*)(g + off));
+                const int valid = (int)(count - off);
+#pragma unroll
+                for (int k = 0; k < 4; k++) {
+                    float a = 2 * k < valid ? h2f(x[k] & 0xFFFFu) : 0.0f;
+                    float b = 2 * k + 1 < valid ? h2f(x[k] >> 16) : 0.0f;
+                    acc = acc + a * a;
+                    acc = acc + b * b;
+                }
+            } else {
+                for (int64_t i = off; i < off + kVec && i < count; i++) {
+                    float a = h2f(ldg<NT>(g + i));
+                    acc = acc + a * a;
+                }
+            }
+        }
+    } else {
+        const float* g = (const float*)r.g;
+        for (int64_t done = 0; done < count; done += kNormGroup) {
+            const int64_t off = done + (int64_t)tid * kVec;
+            if (aligned && off + kVec <= count) {
+                f32x4 x0 = ldg<NT>((const f32x4*)(g + off)), x1 = ldg<NT>((const f32x4*)(g + off) + 1);
+#pragma unroll
+                for (int k = 0; k < 4; k++) acc = acc + x0[k] * x0[k];
+#pragma unroll
+                for (int k = 0; k < 4; k++) acc = acc + x1[k] * x1[k];
+            } else if (aligned && off < count) {
+                // partial last group, as above; the second 16-byte granule is only read if it starts inside
+                const int valid = (int)(count - off);
+                f32x4 x0 = ldg<NT>((const f32x4*)(g + off)), x1 = {0.0f, 0.0f, 0.0f, 0.0f};
+                if (valid > 4) x1 = ldg<NT>((const f32x4*)(g + off) + 1);
+#pragma unroll
+                for (int k = 0; k < 4; k++) { const float a = k < valid ? x0[k] : 0.0f; acc = acc + a * a; }
+#pragma unroll
+                for (int k = 0; k < 4; k++) { const float a = 4 + k < valid ? x1[k] : 0.0f; acc = acc + a * a; }
+            } else {
+                for (int64_t i = off; i < off + kVec && i < count; i++) {
+                    float a = ldg<NT>(g + i);
+                    acc = acc + a * a;
+                }
+            }
+        }
+    }
+    return acc;
+}
+
+// Step 1, general form: one workgroup of BLOCK lanes per chunk (512 lanes with two 128-bit reads each measured
+// 7.3 TB/s as a stand-alone stream, 256 lanes with four 6.95).
 // POOLS: the chunks come from `pools` (two flat buffers passed by value) instead of the table `recs`.
-// PACK > 1 (only with BLOCK = 64, i.e. 512-element chunks): the workgroup has PACK wavefronts and each takes
-// a chunk of its own, PACK consecutive chunks per workgroup.  A list of thousands of small tensors has tens of
-// thousands of such chunks, and one single-wavefront workgroup per chunk is bound by the rate at which
-// workgroups are dispatched; the sum inside a chunk and its slot are the same either way.
-template <bool NT, int BLOCK, bool POOLS = false, int PACK = 1>
+// PACK > 1 (only with BLOCK = 64, i.e. 512-element chunks; kept for comparison): the workgroup has PACK wavefronts
+// and each takes a chunk of its own.
+// FUSED (chunks of 1,024 elements and more): the workgroup that finishes last also runs step 3.
+template <bool NT, int BLOCK, bool POOLS, int PACK, bool FUSED>
 __global__ __launch_bounds__(BLOCK * PACK) void sumsq_partials_kernel(
-    const ChunkRec* __restrict__ recs, PoolPair pools, int64_t n_chunks, double* __restrict__ partials)
+    const ChunkRec* __restrict__ recs, PoolPair pools, int64_t n_chunks, double* partials, NormTail tail)
 {
     static_assert(PACK == 1 || BLOCK == 64, "several chunks per workgroup only with one wavefront per chunk");
-    constexpr int kNormGroup = BLOCK * kVec;
+    static_assert(!FUSED || (PACK == 1 && BLOCK >= 128), "512-element chunks have a kernel of their own");
     __shared__ float wave_sum[BLOCK / 64];
     // which of the workgroup's PACK chunks: the wavefront's number, made known to the compiler as uniform
     // across the wavefront so that the chunk's record is still fetched with scalar loads
@@ -593,91 +815,7 @@ __global__ __launch_bounds__(BLOCK * PACK) void sumsq_partials_kernel(
         ChunkRec r;
         if constexpr (POOLS) r = pool_chunk(pools, c);
         else r = recs[c];
-        const int64_t count = r.count;
-        const bool aligned = ((r.flags >> kValignShift) & 0xF) >= 8;
-
-        float acc = 0.0f;
-        if (r.flags & RLX_TENSOR_FROZEN) {
-            // gradients of a frozen tensor count as zero (the reference clears them before the norm)
-        } else if (!(r.flags & kF32)) {
-            const uint16_t* g = (const uint16_t*)r.g;
-            int64_t done = 0;
-            if (aligned) {
-                for (; done + 2 * (int64_t)kNormGroup <= count; done += 2 * (int64_t)kNormGroup) {
-                    u32x4 x[2];
-#pragma unroll
-                    for (int j = 0; j < 2; j++)
-                        x[j] = ldg<NT>((const u32x4*)(g + done + (int64_t)(j * BLOCK + tid) * kVec));
-#pragma unroll
-                    for (int j = 0; j < 2; j++) {
-#pragma unroll
-                        for (int k = 0; k < 4; k++) {
-                            float a = h2f(x[j][k] & 0xFFFFu), b = h2f(x[j][k] >> 16);
-                            acc = acc + a * a;
-                            acc = acc + b * b;
-                        }
-                    }
-                }
-            }
-            for (; done < count; done += kNormGroup) {
-                const int64_t off = done + (int64_t)tid * kVec;
-                if (aligned && off + kVec <= count) {
-                    u32x4 x = ldg<NT>((const u32x4*)(g + off));
-#pragma unroll
-                    for (int k = 0; k < 4; k++) {
-                        float a = h2f(x[k] & 0xFFFFu), b = h2f(x[k] >> 16);
-                        acc = acc + a * a;
-                        acc = acc + b * b;
-                    }
-                } else if (aligned && off < count) {
-                    // the tensor's last, partial group: its 16-byte granule starts inside the tensor, so one
-                    // aligned load cannot leave the tensor's last page; what lies beyond the end is read but
-                    // counts as zero (acc + 0 leaves a sum of squares as it is).  Element by element this
-                    // lane would wait for up to seven loads one after another, and its workgroup with it.
-                    u32x4 x = ldg<NT>((const u32x4*)(g + off));
-                    const int valid = (int)(count - off);
-#pragma unroll
-                    for (int k = 0; k < 4; k++) {
-                        float a = 2 * k < valid ? h2f(x[k] & 0xFFFFu) : 0.0f;
-                        float b = 2 * k + 1 < valid ? h2f(x[k] >> 16) : 0.0f;
-                        acc = acc + a * a;
-                        acc = acc + b * b;
-                    }
-                } else {
-                    for (int64_t i = off; i < off + kVec && i < count; i++) {
-                        float a = h2f(ldg<NT>(g + i));
-                        acc = acc + a * a;
-                    }
-                }
-            }
-        } else {
-            const float* g = (const float*)r.g;
-            for (int64_t done = 0; done < count; done += kNormGroup) {
-                const int64_t off = done + (int64_t)tid * kVec;
-                if (aligned && off + kVec <= count) {
-                    f32x4 x0 = ldg<NT>((const f32x4*)(g + off)), x1 = ldg<NT>((const f32x4*)(g + off) + 1);
-#pragma unroll
-                    for (int k = 0; k < 4; k++) acc = acc + x0[k] * x0[k];
-#pragma unroll
-                    for (int k = 0; k < 4; k++) acc = acc + x1[k] * x1[k];
-                } else if (aligned && off < count) {
-                    // partial last group, as above; the second 16-byte granule is only read if it starts inside
-                    const int valid = (int)(count - off);
-                    f32x4 x0 = ldg<NT>((const f32x4*)(g + off)), x1 = {0.0f, 0.0f, 0.0f, 0.0f};
-                    if (valid > 4) x1 = ldg<NT>((const f32x4*)(g + off) + 1);
-#pragma unroll
-                    for (int k = 0; k < 4; k++) { const float a = k < valid ? x0[k] : 0.0f; acc = acc + a * a; }
-#pragma unroll
-                    for (int k = 0; k < 4; k++) { const float a = 4 + k < valid ? x1[k] : 0.0f; acc = acc + a * a; }
-                } else {
-                    for (int64_t i = off; i < off + kVec && i < count; i++) {
-                        float a = ldg<NT>(g + i);
-                        acc = acc + a * a;
-                    }
-                }
-            }
-        }
-
+        float acc = chunk_lane_sumsq<NT, BLOCK>(r, tid);
 #pragma unroll
         for (int mask = 32; mask >= 1; mask >>= 1) acc = acc + __shfl_xor(acc, mask, 64);
         if constexpr (BLOCK == 64) {
@@ -695,22 +833,35 @@ __global__ __launch_bounds__(BLOCK * PACK) void sumsq_partials_kernel(
             __syncthreads();
         }
     }
+
+    if constexpr (FUSED) {
+        __shared__ double tree[kFinalBlock];
+        __shared__ int last_flag;
+        if (last_workgroup(tail.tickets, &last_flag)) {
+            const double sum_sq = fixed_order_sum<BLOCK, 16 * BLOCK / kFinalBlock, true>(tail.values, tail.n_values, tree,
+                                                                                       (int)threadIdx.x);
+            if (threadIdx.x == 0) write_norm_result(sum_sq, tail.max_norm, tail.out);
+        }
+    }
 }
 
-// Norm pass 1 for 512-element chunks (lists of thousands of small tensors): a chunk is at most one 8-element
+// Steps 1 and 2 for 512-element chunks (lists of thousands of small tensors): a chunk is at most one 8-element
 // group per lane of one wavefront, so a wavefront takes CPW consecutive chunks at once (records and data of all
-// of them requested before the first is used) and a workgroup of WAVES wavefronts WAVES * CPW chunks.  With one
-// chunk per wavefront the pass is bound by latency: record, data, butterfly, one after another, for each of
-// tens of thousands of chunks.  The sum inside a chunk and its slot are those of the general kernel above with
-// BLOCK = 64 (lane t adds its group's elements in order, xor butterfly), so the results are the same bits.
-template <bool NT, bool POOLS, int WAVES, int CPW>
+// of them requested before the first is used) and a workgroup of WAVES wavefronts WAVES * CPW chunks, a whole
+// number of groups.  With one chunk per wavefront the pass is bound by latency: record, data, butterfly, one
+// after another, for each of tens of thousands of chunks.  The sum inside a chunk and its slot are those of the
+// general kernel above with BLOCK = 64 (lane t adds its group's elements in order, xor butterfly).
+// FUSED: the workgroup that finishes last also runs step 3 over the group partials.
+template <bool NT, bool POOLS, int WAVES, int CPW, bool FUSED>
 __global__ __launch_bounds__(64 * WAVES) void sumsq_small_chunks_kernel(
-    const ChunkRec* __restrict__ recs, PoolPair pools, int64_t n_chunks, double* __restrict__ partials)
+    const ChunkRec* __restrict__ recs, PoolPair pools, int64_t n_chunks, double* partials, double* groups, NormTail tail)
 {
+    constexpr int PER_WG = WAVES * CPW, GROUPS_PER_WG = PER_WG / kGroupChunks;
+    static_assert(PER_WG % kGroupChunks == 0, "a workgroup covers whole groups of chunks");
+    __shared__ double chunk_sum[PER_WG];
     const int lane = threadIdx.x & 63;
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));    // uniform: records by scalar loads
     const int64_t first = ((int64_t)blockIdx.x * WAVES + wave) * CPW;
-    if (first >= n_chunks) return;
 
     const char* g[CPW];
     int valid[CPW];          // elements of chunk j that belong to this lane's group (0..8)
@@ -726,7 +877,7 @@ __global__ __launch_bounds__(64 * WAVES) void sumsq_small_chunks_kernel(
         }
         g[j] = (const char*)r.g;
         f32[j] = (r.flags & kF32) != 0;
-        fast[j] = ((r.flags >> kValignShift) & 0xF) >= 8;
+        fast[j] = ((r.flags >> kGalignShift) & 0xF) >= 8;
         int left = (r.flags & RLX_TENSOR_FROZEN) ? 0 : (int)r.count - lane * kVec;   // a frozen tensor counts as zero
         valid[j] = left < 0 ? 0 : left > kVec ? kVec : left;
     }
@@ -777,49 +928,54 @@ __global__ __launch_bounds__(64 * WAVES) void sumsq_small_chunks_kernel(
         }
 #pragma unroll
         for (int mask = 32; mask >= 1; mask >>= 1) acc = acc + __shfl_xor(acc, mask, 64);
-        if (lane == 0 && first + j < n_chunks) partials[first + j] = (double)acc;
+        if (lane == 0) {
+            const bool exists = first + j < n_chunks;
+            if (exists) partials[first + j] = (double)acc;
+            chunk_sum[wave * CPW + j] = exists ? (double)acc : 0.0;     // +0.0 leaves the group's sum as it is
+        }
+    }
+    __syncthreads();
+    if (threadIdx.x < GROUPS_PER_WG) {
+        const int64_t grp = (int64_t)blockIdx.x * GROUPS_PER_WG + threadIdx.x;
+        if (grp * kGroupChunks < n_chunks) {
+            double total = 0.0;
+#pragma unroll
+            for (int k = 0; k < kGroupChunks; k++) total += chunk_sum[threadIdx.x * kGroupChunks + k];
+            groups[grp] = total;
+        }
+    }
+    if constexpr (FUSED) {
+        __shared__ double tree[kFinalBlock];
+        __shared__ int last_flag;
+        if (last_workgroup(tail.tickets, &last_flag)) {
+            const double sum_sq = fixed_order_sum<64 * WAVES, 16 * 64 * WAVES / kFinalBlock, true>(
+                tail.values, tail.n_values, tree, (int)threadIdx.x);
+            if (threadIdx.x == 0) write_norm_result(sum_sq, tail.max_norm, tail.out);
+        }
     }
 }
 
-// Norm pass 2: one workgroup, fixed order.  Thread t adds partials t, t+1024, ... in FP64,
-// then a halving tree through LDS.  Writes the sum, the norm and the clip scale
-// (trainer.h:341-345: strict '>' and +1e-6f in the denominator).
+// Step 2 as a launch of its own, for the forms of step 1 that have fewer than 16 chunks per workgroup (kept for
+// comparison): one lane per group adds the group's chunk partials in index order.
+__global__ __launch_bounds__(256) void sumsq_group_kernel(const double* __restrict__ partials, int64_t n_chunks,
+                                                          double* __restrict__ groups)
+{
+    const int64_t grp = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t first = grp * kGroupChunks;
+    if (first >= n_chunks) return;
+    double total = 0.0;
+    for (int k = 0; k < kGroupChunks; k++) total += first + k < n_chunks ? partials[first + k] : 0.0;
+    groups[grp] = total;
+}
+
+// Step 3 as a launch of its own: one workgroup of 1,024 lanes.  BATCH: rounds of loads in flight per lane.
 template <int BATCH>
 __global__ __launch_bounds__(kFinalBlock) void sumsq_final_kernel(
-    const double* __restrict__ partials, int64_t n_partials, float max_norm, NormResult* __restrict__ out)
+    const double* __restrict__ values, int64_t n_values, float max_norm, NormResult* __restrict__ out)
 {
-    __shared__ double acc[kFinalBlock];
-    const int tid = threadIdx.x;
-    double a = 0.0;
-    int64_t i = tid;
-    // BATCH independent loads in flight, added in index order: the same sum as one at a time.  Slots beyond
-    // the end read as +0.0, which leaves a sum of squares (never negative zero) unchanged bit for bit; without
-    // them the last few partials of every lane would each cost a round trip of their own.
-    for (; i < n_partials; i += BATCH * (int64_t)kFinalBlock) {
-        double x[BATCH];
-#pragma unroll
-        for (int k = 0; k < BATCH; k++) {
-            const int64_t j = i + k * (int64_t)kFinalBlock;
-            x[k] = j < n_partials ? partials[j] : 0.0;
-        }
-#pragma unroll
-        for (int k = 0; k < BATCH; k++) a += x[k];
-    }
-    acc[tid] = a;
-    __syncthreads();
-    for (int s = kFinalBlock / 2; s >= 1; s >>= 1) {
-        if (tid < s) acc[tid] = acc[tid] + acc[tid + s];
-        __syncthreads();
-    }
-    if (tid == 0) {
-        const double sum_sq = acc[0];
-        const float norm = __builtin_sqrtf((float)sum_sq);
-        float scale = 1.0f;
-        if (norm > max_norm) scale = max_norm / (norm + 1e-6f);
-        out->sum_sq = sum_sq;
-        out->norm = norm;
-        out->scale = scale;
-    }
+    __shared__ double tree[kFinalBlock];
+    const double sum_sq = fixed_order_sum<kFinalBlock, BATCH, false>(values, n_values, tree, (int)threadIdx.x);
+    if (threadIdx.x == 0) write_norm_result(sum_sq, max_norm, out);
 }
 
 // In-place scale of the gradients (trainer.h:136-145).  Exactly 1.0f: nothing is touched.
@@ -842,7 +998,7 @@ __global__ __launch_bounds__(BLOCK) void scale_group_kernel(
     const int64_t count = r.count;
     const int64_t off = base + (int64_t)threadIdx.x * kVec;
     if (off >= count) return;
-    const bool aligned = ((r.flags >> kValignShift) & 0xF) >= 8;
+    const bool aligned = ((r.flags >> kGalignShift) & 0xF) >= 8;
     if (!(r.flags & kF32)) {
         uint16_t* g = (uint16_t*)r.g;
         if (aligned && off + kVec <= count) {
@@ -924,17 +1080,19 @@ __global__ __launch_bounds__(256) void fp16_to_fp32_kernel(float* __restrict__ d
 }
 
 // After an update that read the current entry of a plan's step table: move on to the next entry, so that the
-// next (replayed) update reads new hyper-parameters without the host.  Beyond the end of the table the last
-// entry stays current; *taken counts the scheduled steps so far, saturating at n.
-__global__ __launch_bounds__(64) void schedule_advance_kernel(const rlx_step_params* __restrict__ table, int64_t n,
-                                                              int64_t* __restrict__ taken,
-                                                              rlx_step_params* __restrict__ current)
+// next (replayed) update reads new hyper-parameters without the host.  The launch names only the header, whose
+// address never changes while the plan lives; the table's address and length are read from it at run time, so a
+// recorded launch follows every later upload, whatever its length.  Beyond the end of the table the last entry
+// stays current; `taken` counts the scheduled steps so far, saturating at the length, and `overrun` counts the
+// updates that ran with the last entry again because the table had been used up.
+__global__ __launch_bounds__(64) void schedule_advance_kernel(SchedHeader* __restrict__ hdr)
 {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
-    int64_t next = *taken + 1;
-    if (next < n) *current = table[next];
-    if (next > n) next = n;
-    *taken = next;
+    const int64_t n = hdr->len, done = hdr->taken;
+    if (done >= n) { hdr->overrun = hdr->overrun + 1; return; }      // this update read a used-up table
+    const int64_t next = done + 1;
+    if (next < n) hdr->current = hdr->table[next];
+    hdr->taken = next;
 }
 
 // Zero fill as a kernel (a memset node recorded into a HIP graph is not reliable on every
@@ -1029,6 +1187,9 @@ struct Tuning {
                                             // 2 = thirty-two (four per wavefront, the default), 3 = sixteen
     std::atomic<int64_t> convert_variant{0};
     std::atomic<int64_t> final_batch{0};    // loads in flight per lane in the second pass of the norm; 0 = by the number of partials
+    std::atomic<int64_t> norm_fused{2};     // the fixed-order sum of the partials: 0 = always a second launch, 1 = by the
+                                            // workgroup of the first launch that finishes last whenever that launch
+                                            // has at most 8,192 workgroups, 2 = that up to 4,096 workgroups (default)
 } g_tuning;
 
 constexpr int kNumUpdateVariants = 17;
@@ -1102,6 +1263,14 @@ ChunkRec make_rec(const rlx_tensor_desc& d, int64_t start, int64_t count) {
         }
     }
     r.flags |= valign << kValignShift;
+    uint32_t galign = 1;
+    for (uint32_t e = 8; e > 1; e >>= 1) {
+        if (is_aligned(r.g, e * es)) {
+            galign = e;
+            break;
+        }
+    }
+    r.flags |= galign << kGalignShift;
     return r;
 }
 
@@ -1123,8 +1292,12 @@ hipError_t launch_variant(const ChunkRec* recs, const ChunkRec& single, int64_t 
     for (int64_t first = 0; first < n_tiles; first += kMaxTilesPerLaunch) {
         int64_t here = n_tiles - first < kMaxTilesPerLaunch ? n_tiles - first : kMaxTilesPerLaunch;
         here = (here + 8 * K - 1) / (8 * K) * (8 * K);   // whole swizzle groups; the excess exits at once
-        adamw_tile_kernel<E, BLOCK, K, SINGLE, SP, PH, NTL><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(
-            recs, single, single_n, first, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
+        if (norm)
+            adamw_tile_kernel<E, BLOCK, K, SINGLE, SP, PH, NTL, true><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(
+                recs, single, single_n, first, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
+        else
+            adamw_tile_kernel<E, BLOCK, K, SINGLE, SP, PH, NTL, false><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(
+                recs, single, single_n, first, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -1156,8 +1329,12 @@ hipError_t launch_persistent(const ChunkRec* recs, int64_t n_chunks, int chunk_l
     int64_t grid = (int64_t)compute_units() * kPersistentPerCU;
     const int64_t need = (n_tiles + kPersistentWaves - 1) / kPersistentWaves;
     if (grid > need) grid = need;
-    adamw_persistent_kernel<E, kPersistentWaves, SP, NTL><<<dim3((unsigned)grid), dim3(64 * kPersistentWaves), 0, s>>>(
-        recs, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
+    if (norm)
+        adamw_persistent_kernel<E, kPersistentWaves, SP, NTL, true><<<dim3((unsigned)grid), dim3(64 * kPersistentWaves), 0, s>>>(
+            recs, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
+    else
+        adamw_persistent_kernel<E, kPersistentWaves, SP, NTL, false><<<dim3((unsigned)grid), dim3(64 * kPersistentWaves), 0, s>>>(
+            recs, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
     return hipGetLastError();
 }
 
@@ -1166,8 +1343,12 @@ hipError_t launch_per_chunk(const ChunkRec* recs, int64_t n_chunks, const Hyper&
                             const NormResult* norm, uint32_t step_flags, hipStream_t s) {
     for (int64_t first = 0; first < n_chunks; first += kMaxTilesPerLaunch) {
         const int64_t here = n_chunks - first < kMaxTilesPerLaunch ? n_chunks - first : kMaxTilesPerLaunch;
-        adamw_chunk_kernel<8, 256, SP, NTL><<<dim3((unsigned)here), dim3(256), 0, s>>>(recs, first, n_chunks, h, dev_params, norm,
-                                                                               step_flags);
+        if (norm)
+            adamw_chunk_kernel<8, 256, SP, NTL, true><<<dim3((unsigned)here), dim3(256), 0, s>>>(recs, first, n_chunks, h,
+                                                                                         dev_params, norm, step_flags);
+        else
+            adamw_chunk_kernel<8, 256, SP, NTL, false><<<dim3((unsigned)here), dim3(256), 0, s>>>(recs, first, n_chunks, h,
+                                                                                          dev_params, norm, step_flags);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
@@ -1182,15 +1363,20 @@ hipError_t launch_rounds(const ChunkRec* recs, int64_t n_chunks, int chunk_log2,
     const int64_t n_tiles = n_chunks << tpc_log2;
     for (int64_t first = 0; first < n_tiles; first += kMaxTilesPerLaunch) {
         const int64_t here = n_tiles - first < kMaxTilesPerLaunch ? n_tiles - first : kMaxTilesPerLaunch;
-        adamw_rounds_kernel<E, BLOCK, R, 1><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(recs, first, n_tiles, tpc_log2, h,
-                                                                                      dev_params, norm, step_flags);
+        if (norm)
+            adamw_rounds_kernel<E, BLOCK, R, 1, true><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(recs, first, n_tiles, tpc_log2,
+                                                                                            h, dev_params, norm, step_flags);
+        else
+            adamw_rounds_kernel<E, BLOCK, R, 1, false><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(recs, first, n_tiles, tpc_log2,
+                                                                                             h, dev_params, norm, step_flags);
         const hipError_t e = hipGetLastError();
         if (e != hipSuccess) return e;
     }
     return hipSuccess;
 }
 
-// The compiled forms of the update ("update_variant"), by number; 0 is what ships.
+// The compiled forms of the update ("update_variant"), by number; 0 is what ships.  Every kernel has one more,
+// last template argument that the names leave out: false for the plain update, true for the fused-clip one.
 const char* const kVariantNames[kNumUpdateVariants] = {
     "adamw_tile_kernel<2,128,1,*,1,0|1>",      // 0: 2 elements x 128 lanes, sc1 nt stores; loads at once, or two
                                                //    at a time when the step writes four streams
@@ -1305,15 +1491,16 @@ struct rlx_plan {
     // more than kMaxIdleRanges of them (such steps then run over the full table)
     std::vector<std::pair<void*, int64_t>> idle_grads;
     bool idle_by_range;
-    double* d_partials;
+    double* d_partials;      // one allocation: per-chunk partials, then the group partials (one per 16 chunks),
+    double* d_groups;        // then the ticket counters of the norm launch (zero between launches)
+    uint32_t* d_tickets;
     NormResult* d_norm;
     NormResult* h_norm;      // pinned
     // host-free replay: a table of per-step hyper-parameters on the device, the entry that the next scheduled
     // update reads (d_current) and the count of scheduled steps taken (d_taken); all null until a table is uploaded
     rlx_step_params* d_sched;
     int64_t sched_cap, sched_len;
-    rlx_step_params* d_current;
-    int64_t* d_taken;
+    SchedHeader* d_header;
 };
 
 namespace {
@@ -1331,7 +1518,7 @@ int plan_launchable(const rlx_plan* p) {
 }
 
 template <int BLOCK>
-void launch_scale_groups(const rlx_plan* p, hipStream_t s) {
+hipError_t launch_scale_groups(const rlx_plan* p, hipStream_t s) {
     constexpr int TILE = BLOCK * kVec;
     // chunks smaller than one group: one workgroup per chunk, the lanes beyond its end drop out
     const int tpc_log2 = p->chunk_log2 > __builtin_ctz(TILE) ? p->chunk_log2 - __builtin_ctz(TILE) : 0;
@@ -1340,73 +1527,126 @@ void launch_scale_groups(const rlx_plan* p, hipStream_t s) {
         const int64_t here = n_tiles - first < kMaxTilesPerLaunch ? n_tiles - first : kMaxTilesPerLaunch;
         scale_group_kernel<BLOCK><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(p->d_recs, first, n_tiles, tpc_log2,
                                                                              p->d_norm);
+        const hipError_t e = hipGetLastError();
+        if (e != hipSuccess) return e;
     }
+    return hipSuccess;
 }
 
-// Pass 2.  How many loads a lane keeps in flight only changes the speed, not the order of the sum.
-void launch_final(const double* partials, int64_t n, float max_norm, NormResult* result, hipStream_t s) {
+// Step 3 of the norm as a launch of its own.  How many loads a lane keeps in flight only changes the speed, not
+// the order of the sum.
+hipError_t launch_final(const double* values, int64_t n, float max_norm, NormResult* result, hipStream_t s) {
     int64_t batch = g_tuning.final_batch;
-    if (batch == 0) {          // automatic: about as many as a lane has partials to add, so that few slots are empty
+    if (batch == 0) {          // automatic: about as many as a lane has values to add, so that few slots are empty
         const int64_t per_lane = (n + kFinalBlock - 1) / kFinalBlock;
         batch = per_lane <= 8 ? 8 : per_lane <= 16 ? 16 : per_lane <= 32 ? 32 : 40;
     }
-    if (batch == 8) sumsq_final_kernel<8><<<dim3(1), dim3(kFinalBlock), 0, s>>>(partials, n, max_norm, result);
-    else if (batch == 32) sumsq_final_kernel<32><<<dim3(1), dim3(kFinalBlock), 0, s>>>(partials, n, max_norm, result);
-    else if (batch == 40) sumsq_final_kernel<40><<<dim3(1), dim3(kFinalBlock), 0, s>>>(partials, n, max_norm, result);
-    else sumsq_final_kernel<16><<<dim3(1), dim3(kFinalBlock), 0, s>>>(partials, n, max_norm, result);
+    if (batch == 8) sumsq_final_kernel<8><<<dim3(1), dim3(kFinalBlock), 0, s>>>(values, n, max_norm, result);
+    else if (batch == 32) sumsq_final_kernel<32><<<dim3(1), dim3(kFinalBlock), 0, s>>>(values, n, max_norm, result);
+    else if (batch == 40) sumsq_final_kernel<40><<<dim3(1), dim3(kFinalBlock), 0, s>>>(values, n, max_norm, result);
+    else sumsq_final_kernel<16><<<dim3(1), dim3(kFinalBlock), 0, s>>>(values, n, max_norm, result);
+    return hipGetLastError();
 }
 
-// Both passes of the norm over n_chunks chunks (from the table `recs`, or from `pools` if POOLS): one FP64
-// partial per chunk into `partials`, then the fixed-order sum and the clip rule into `result`.
-template <bool POOLS>
-int launch_norm(const ChunkRec* recs, const PoolPair& pools, int64_t n_chunks, int64_t chunk_elems, double* partials,
-                float max_norm, NormResult* result, hipStream_t s) {
-    const int64_t norm_grid = g_tuning.norm_grid, norm_pack = g_tuning.norm_pack;
-    const bool norm_nt = g_tuning.norm_nt != 0;
-    int64_t g = norm_grid > 0 ? norm_grid : n_chunks;
-    if (g > n_chunks) g = n_chunks;
-    if (g > kMaxNormGrid) g = kMaxNormGrid;
-    const dim3 grid((unsigned)g);
-    const int64_t lanes = chunk_elems / kVec < kNormBlock ? chunk_elems / kVec : kNormBlock;
-#define RLX_NORM_LAUNCH(BLOCK)                                                                                       \
-    do {                                                                                                             \
-        if (norm_nt)                                                                                        \
-            sumsq_partials_kernel<true, BLOCK, POOLS><<<grid, dim3(BLOCK), 0, s>>>(recs, pools, n_chunks, partials);  \
-        else                                                                                                         \
-            sumsq_partials_kernel<false, BLOCK, POOLS><<<grid, dim3(BLOCK), 0, s>>>(recs, pools, n_chunks, partials); \
-    } while (0)
-    if (lanes >= 512) RLX_NORM_LAUNCH(512);
-    else if (lanes == 256) RLX_NORM_LAUNCH(256);
-    else if (lanes == 128) RLX_NORM_LAUNCH(128);
-    else if (norm_pack == 0) RLX_NORM_LAUNCH(64);
-    else if (norm_pack == 1) {
-        // 512-element chunks: eight wavefronts per workgroup, one chunk each
-        constexpr int PACK = 8;
-        const dim3 pgrid((unsigned)((g + PACK - 1) / PACK));
-        if (norm_nt)
-            sumsq_partials_kernel<true, 64, POOLS, PACK><<<pgrid, dim3(64 * PACK), 0, s>>>(recs, pools, n_chunks, partials);
+// Where one norm launch reads its chunks and keeps its intermediate sums.
+struct NormWork {
+    const ChunkRec* recs;        // the chunk table, or
+    PoolPair pools;              // two flat buffers by value (POOLS)
+    int64_t n_chunks, chunk_elems;
+    double* partials;            // one per chunk
+    double* groups;              // one per 16 chunks; only used with 512-element chunks
+    uint32_t* tickets;           // kTicketWords words, all zero between launches
+    NormResult* result;
+};
+
+inline int64_t norm_groups(int64_t n_chunks) { return (n_chunks + kGroupChunks - 1) / kGroupChunks; }
+
+// Workgroups up to which the automatic choice ("norm_fused" = 2) lets the last workgroup add the partials.
+constexpr int64_t kAutoFusedWgs = 4096;
+
+template <bool NT, bool POOLS, int BLOCK>
+hipError_t launch_partials(const NormWork& w, int64_t grid, bool fused, const NormTail& tail, hipStream_t s) {
+    if (fused)
+        sumsq_partials_kernel<NT, BLOCK, POOLS, 1, true><<<dim3((unsigned)grid), dim3(BLOCK), 0, s>>>(
+            w.recs, w.pools, w.n_chunks, w.partials, tail);
+    else
+        sumsq_partials_kernel<NT, BLOCK, POOLS, 1, false><<<dim3((unsigned)grid), dim3(BLOCK), 0, s>>>(
+            w.recs, w.pools, w.n_chunks, w.partials, tail);
+    return hipGetLastError();
+}
+
+template <bool NT, bool POOLS, int WAVES, int CPW>
+hipError_t launch_small_chunks(const NormWork& w, int64_t grid, bool fused, const NormTail& tail, hipStream_t s) {
+    if (fused)
+        sumsq_small_chunks_kernel<NT, POOLS, WAVES, CPW, true><<<dim3((unsigned)grid), dim3(64 * WAVES), 0, s>>>(
+            w.recs, w.pools, w.n_chunks, w.partials, w.groups, tail);
+    else
+        sumsq_small_chunks_kernel<NT, POOLS, WAVES, CPW, false><<<dim3((unsigned)grid), dim3(64 * WAVES), 0, s>>>(
+            w.recs, w.pools, w.n_chunks, w.partials, w.groups, tail);
+    return hipGetLastError();
+}
+
+// The whole norm: per-chunk partials (and group partials for 512-element chunks), then the fixed-order sum and
+// the clip rule into w.result, as the tail of the same launch or as a second one ("norm_fused").
+template <bool NT, bool POOLS>
+int launch_norm_nt(const NormWork& w, float max_norm, hipStream_t s) {
+    const int64_t norm_grid = g_tuning.norm_grid, norm_pack = g_tuning.norm_pack, norm_fused = g_tuning.norm_fused;
+    const int64_t lanes = w.chunk_elems / kVec < kNormBlock ? w.chunk_elems / kVec : kNormBlock;
+    const bool grouped = lanes == 64;
+    NormTail tail;
+    tail.values = grouped ? w.groups : w.partials;
+    tail.n_values = grouped ? norm_groups(w.n_chunks) : w.n_chunks;
+    tail.max_norm = max_norm;
+    tail.out = w.result;
+    tail.tickets = w.tickets;
+    const auto want_fused = [&](int64_t grid) {
+        return grid <= kMaxFusedWgs && (norm_fused == 1 || (norm_fused == 2 && grid <= kAutoFusedWgs));
+    };
+    bool fused = false;
+    hipError_t e = hipSuccess;
+    if (!grouped) {
+        int64_t g = norm_grid > 0 ? norm_grid : w.n_chunks;
+        if (g > w.n_chunks) g = w.n_chunks;
+        if (g > kMaxNormGrid) g = kMaxNormGrid;
+        fused = want_fused(g);
+        if (lanes >= 512) e = launch_partials<NT, POOLS, 512>(w, g, fused, tail, s);
+        else if (lanes == 256) e = launch_partials<NT, POOLS, 256>(w, g, fused, tail, s);
+        else e = launch_partials<NT, POOLS, 128>(w, g, fused, tail, s);
+    } else if (norm_pack == 0 || norm_pack == 1) {
+        // 512-element chunks, one per workgroup or eight (a wavefront each): fewer chunks per workgroup than a
+        // group has, so the group partials take a launch of their own (both kept for comparison)
+        int64_t g = norm_grid > 0 ? norm_grid : w.n_chunks;
+        if (g > w.n_chunks) g = w.n_chunks;
+        if (g > kMaxNormGrid) g = kMaxNormGrid;
+        if (norm_pack == 0)
+            sumsq_partials_kernel<NT, 64, POOLS, 1, false><<<dim3((unsigned)g), dim3(64), 0, s>>>(
+                w.recs, w.pools, w.n_chunks, w.partials, tail);
         else
-            sumsq_partials_kernel<false, 64, POOLS, PACK><<<pgrid, dim3(64 * PACK), 0, s>>>(recs, pools, n_chunks, partials);
+            sumsq_partials_kernel<NT, 64, POOLS, 8, false><<<dim3((unsigned)((g + 7) / 8)), dim3(512), 0, s>>>(
+                w.recs, w.pools, w.n_chunks, w.partials, tail);
+        e = hipGetLastError();
+        if (e == hipSuccess) {
+            sumsq_group_kernel<<<dim3((unsigned)((tail.n_values + 255) / 256)), dim3(256), 0, s>>>(w.partials, w.n_chunks,
+                                                                                                 w.groups);
+            e = hipGetLastError();
+        }
     } else {
         // 512-element chunks, the default: eight wavefronts per workgroup, four (or two) chunks each
-#define RLX_SMALL(W, C)                                                                                          \
-    do {                                                                                                         \
-        const int64_t per_wg = (W) * (C);                                                                        \
-        const dim3 pgrid((unsigned)((n_chunks + per_wg - 1) / per_wg));                                          \
-        if (norm_nt)                                                                                    \
-            sumsq_small_chunks_kernel<true, POOLS, W, C><<<pgrid, dim3(64 * (W)), 0, s>>>(recs, pools, n_chunks, partials);  \
-        else                                                                                                     \
-            sumsq_small_chunks_kernel<false, POOLS, W, C><<<pgrid, dim3(64 * (W)), 0, s>>>(recs, pools, n_chunks, partials); \
-    } while (0)
-        if (norm_pack == 3) RLX_SMALL(8, 2);
-        else RLX_SMALL(8, 4);
-#undef RLX_SMALL
+        const int64_t per_wg = norm_pack == 3 ? 16 : 32;
+        const int64_t g = (w.n_chunks + per_wg - 1) / per_wg;
+        if (g > kMaxNormGrid) return RLX_ERR_TOO_LARGE;
+        fused = want_fused(g);
+        if (norm_pack == 3) e = launch_small_chunks<NT, POOLS, 8, 2>(w, g, fused, tail, s);
+        else e = launch_small_chunks<NT, POOLS, 8, 4>(w, g, fused, tail, s);
     }
-#undef RLX_NORM_LAUNCH
-    RLX_HIP(hipGetLastError());
-    launch_final(partials, n_chunks, max_norm, result, s);
-    RLX_HIP(hipGetLastError());
+    if (e == hipSuccess && !fused) e = launch_final(tail.values, tail.n_values, max_norm, w.result, s);
+    if (e != hipSuccess) return hip_fail(e, "norm kernel launch");
     return RLX_OK;
+}
+
+template <bool POOLS>
+int launch_norm(const NormWork& w, float max_norm, hipStream_t s) {
+    return g_tuning.norm_nt != 0 ? launch_norm_nt<true, POOLS>(w, max_norm, s) : launch_norm_nt<false, POOLS>(w, max_norm, s);
 }
 
 // The update launch of a plan.  Frozen and grad-only chunks have nothing to update, and a workgroup that only
@@ -1452,7 +1692,7 @@ const char* rlx_status_string(int status) {
 
 const char* rlx_last_hip_error(void) { return g_hip_error; }
 
-int rlx_version(void) { return 108; }
+int rlx_version(void) { return 109; }
 
 int rlx_adamw_fp16(float* master_w, uint16_t* model_w, const uint16_t* grad, float* m, float* v, int64_t n,
                    float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -1512,8 +1752,8 @@ int rlx_scale_f32(float* x, float scale, int64_t n, void* stream) {
         const int64_t here = lanes - first < per_launch ? lanes - first : per_launch;
         scale_f32_kernel<<<dim3((unsigned)((here + 255) / 256)), dim3(256), 0, (hipStream_t)stream>>>(
             x + first * 4, scale, n - first * 4, is_aligned(x, 16) ? 1 : 0);
+        RLX_HIP(hipGetLastError());
     }
-    RLX_HIP(hipGetLastError());
     return RLX_OK;
 }
 
@@ -1586,12 +1826,18 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
                 p->idle_by_range = false;
         }
     }
-    p->d_recs = nullptr; p->d_active = nullptr; p->n_active = 0; p->d_partials = nullptr; p->d_norm = nullptr; p->h_norm = nullptr;
-    p->d_sched = nullptr; p->sched_cap = 0; p->sched_len = 0; p->d_current = nullptr; p->d_taken = nullptr;
+    p->d_recs = nullptr; p->d_active = nullptr; p->n_active = 0; p->d_partials = nullptr; p->d_groups = nullptr; p->d_tickets = nullptr; p->d_norm = nullptr; p->h_norm = nullptr;
+    p->d_sched = nullptr; p->sched_cap = 0; p->sched_len = 0; p->d_header = nullptr;
 
     hipError_t e = hipGetDevice(&p->device);
     if (e == hipSuccess) e = hipMalloc((void**)&p->d_recs, sizeof(ChunkRec) * (size_t)n_chunks);
-    if (e == hipSuccess) e = hipMalloc((void**)&p->d_partials, sizeof(double) * (size_t)n_chunks);
+    const size_t n_sums = (size_t)n_chunks + (size_t)norm_groups(n_chunks);
+    if (e == hipSuccess) e = hipMalloc((void**)&p->d_partials, sizeof(double) * n_sums + sizeof(uint32_t) * (size_t)kTicketWords);
+    if (e == hipSuccess) {
+        p->d_groups = p->d_partials + n_chunks;
+        p->d_tickets = (uint32_t*)(p->d_partials + n_sums);
+        e = hipMemset(p->d_tickets, 0, sizeof(uint32_t) * (size_t)kTicketWords);
+    }
     if (e == hipSuccess) e = hipMalloc((void**)&p->d_norm, sizeof(NormResult));
     if (e == hipSuccess) e = hipHostMalloc((void**)&p->h_norm, sizeof(NormResult), hipHostMallocDefault);
     if (e == hipSuccess) e = hipMemcpy(p->d_recs, recs.data(), sizeof(ChunkRec) * (size_t)n_chunks, hipMemcpyHostToDevice);
@@ -1635,7 +1881,7 @@ int rlx_plan_destroy(rlx_plan* p) {
     if (p->d_norm && (e = hipFree(p->d_norm)) != hipSuccess && first == hipSuccess) first = e;
     if (p->h_norm && (e = hipHostFree(p->h_norm)) != hipSuccess && first == hipSuccess) first = e;
     if (p->d_sched && (e = hipFree(p->d_sched)) != hipSuccess && first == hipSuccess) first = e;
-    if (p->d_current && (e = hipFree(p->d_current)) != hipSuccess && first == hipSuccess) first = e;
+    if (p->d_header && (e = hipFree(p->d_header)) != hipSuccess && first == hipSuccess) first = e;
     p->magic = 0;
     delete p;
     return first == hipSuccess ? RLX_OK : hip_fail(first, "rlx_plan_destroy");
@@ -1650,10 +1896,11 @@ const double* rlx_plan_partials_device_ptr(const rlx_plan* p) { return plan_ok(p
 int rlx_plan_grad_norm(rlx_plan* p, float max_norm, void* stream) {
     const int ready = plan_launchable(p);
     if (ready != RLX_OK) return ready;
-    PoolPair none;
-    memset(&none, 0, sizeof(none));
-    return launch_norm<false>(p->d_recs, none, p->n_chunks, p->chunk_elems, p->d_partials, max_norm, p->d_norm,
-                              (hipStream_t)stream);
+    NormWork w;
+    memset(&w, 0, sizeof(w));
+    w.recs = p->d_recs; w.n_chunks = p->n_chunks; w.chunk_elems = p->chunk_elems;
+    w.partials = p->d_partials; w.groups = p->d_groups; w.tickets = p->d_tickets; w.result = p->d_norm;
+    return launch_norm<false>(w, max_norm, (hipStream_t)stream);
 }
 
 /* Device address of the static scratch array on the current device, resolved once per device. */
@@ -1694,16 +1941,20 @@ int rlx_grad_norm_static(const uint16_t* half_grads, int64_t n_half, const float
     pp.flags_half = make_rec(d, 0, 0).flags;
     d.grad = const_cast<float*>(float_grads); d.dtype = RLX_DTYPE_F32;
     pp.flags_float = make_rec(d, 0, 0).flags;
-    double* partials = nullptr;
-    const int st = static_scratch(&partials);
+    double* base = nullptr;
+    const int st = static_scratch(&base);
     if (st != RLX_OK) return st;
     if (n_chunks == 0) {      // nothing to add up: sum 0, norm 0, scale by the rule
-        launch_final(partials, 0, max_norm, (NormResult*)result_dev, (hipStream_t)stream);
-        RLX_HIP(hipGetLastError());
+        RLX_HIP(launch_final(base, 0, max_norm, (NormResult*)result_dev, (hipStream_t)stream));
         return RLX_OK;
     }
-    return launch_norm<true>(nullptr, pp, n_chunks, chunk_elems, partials, max_norm, (NormResult*)result_dev,
-                             (hipStream_t)stream);
+    NormWork w;
+    memset(&w, 0, sizeof(w));
+    w.pools = pp; w.n_chunks = n_chunks; w.chunk_elems = chunk_elems;
+    w.partials = base; w.groups = base + kStaticMaxPartials;
+    w.tickets = (uint32_t*)(base + kStaticMaxPartials + kStaticMaxGroups);
+    w.result = (NormResult*)result_dev;
+    return launch_norm<true>(w, max_norm, (hipStream_t)stream);
 }
 
 int rlx_plan_norm_read(rlx_plan* p, float* norm, float* scale, double* sum_sq, void* stream) {
@@ -1721,8 +1972,7 @@ int rlx_plan_norm_read(rlx_plan* p, float* norm, float* scale, double* sum_sq, v
 int rlx_plan_scale_grads(rlx_plan* p, void* stream) {
     const int ready = plan_launchable(p);
     if (ready != RLX_OK) return ready;
-    launch_scale_groups<kScaleBlock>(p, (hipStream_t)stream);
-    RLX_HIP(hipGetLastError());
+    RLX_HIP(launch_scale_groups<kScaleBlock>(p, (hipStream_t)stream));
     return RLX_OK;
 }
 
@@ -1759,24 +2009,36 @@ int rlx_plan_schedule_upload(rlx_plan* p, const rlx_step_params* steps, int64_t 
                                    steps[i].bias_correction1, steps[i].bias_correction2);
         if (st != RLX_OK) return st;
     }
-    // scheduled updates already in the stream still read the old table
-    RLX_HIP(hipStreamSynchronize((hipStream_t)stream));
-    if (!p->d_current) {
-        // one small allocation: the current entry (28 bytes, padded to 32) followed by the step count
-        RLX_HIP(hipMalloc((void**)&p->d_current, 40));
-        p->d_taken = (int64_t*)((char*)p->d_current + 32);
-    }
+    (void)stream;
+    // Scheduled updates of this plan that are still running, on whatever stream (replays of a recorded step
+    // included), read the header and the old table: wait for the whole device, not only for `stream`.
+    RLX_HIP(hipDeviceSynchronize());
+    if (!p->d_header) RLX_HIP(hipMalloc((void**)&p->d_header, sizeof(SchedHeader)));   // address fixed from here on
+    rlx_step_params* table = p->d_sched;
+    rlx_step_params* retired = nullptr;
     if (n_steps > p->sched_cap) {
-        if (p->d_sched) RLX_HIP(hipFree(p->d_sched));
-        p->d_sched = nullptr; p->sched_cap = 0;
-        RLX_HIP(hipMalloc((void**)&p->d_sched, sizeof(rlx_step_params) * (size_t)n_steps));
-        p->sched_cap = n_steps;
+        // A longer table gets a new allocation.  Recorded launches hold the header's address, never the table's,
+        // and nothing is running, so the old table can go once the header names the new one.
+        RLX_HIP(hipMalloc((void**)&table, sizeof(rlx_step_params) * (size_t)n_steps));
+        retired = p->d_sched;
     }
-    const int64_t zero = 0;
-    RLX_HIP(hipMemcpy(p->d_sched, steps, sizeof(rlx_step_params) * (size_t)n_steps, hipMemcpyHostToDevice));
-    RLX_HIP(hipMemcpy(p->d_current, steps, sizeof(rlx_step_params), hipMemcpyHostToDevice));
-    RLX_HIP(hipMemcpy(p->d_taken, &zero, sizeof(zero), hipMemcpyHostToDevice));
+    hipError_t e = hipMemcpy(table, steps, sizeof(rlx_step_params) * (size_t)n_steps, hipMemcpyHostToDevice);
+    if (e == hipSuccess) {
+        SchedHeader h;
+        memset(&h, 0, sizeof(h));
+        h.current = steps[0];
+        h.table = table;
+        h.len = n_steps;
+        e = hipMemcpy(p->d_header, &h, sizeof(h), hipMemcpyHostToDevice);
+    }
+    if (e != hipSuccess) {
+        // the header still names the old table (or none): leave the plan as it was
+        if (table != p->d_sched) (void)hipFree(table);
+        return hip_fail(e, "rlx_plan_schedule_upload");
+    }
+    if (table != p->d_sched) { p->d_sched = table; p->sched_cap = n_steps; }
     p->sched_len = n_steps;
+    if (retired) RLX_HIP(hipFree(retired));
     return RLX_OK;
 }
 
@@ -1787,10 +2049,9 @@ int rlx_plan_adamw_scheduled(rlx_plan* p, int step_flags, void* stream) {
     if (ready != RLX_OK) return ready;
     Hyper h;
     memset(&h, 0, sizeof(h));
-    const int st = plan_update(p, h, p->d_current, step_flags, (hipStream_t)stream);
+    const int st = plan_update(p, h, &p->d_header->current, step_flags, (hipStream_t)stream);
     if (st != RLX_OK) return st;
-    schedule_advance_kernel<<<dim3(1), dim3(64), 0, (hipStream_t)stream>>>(p->d_sched, p->sched_len, p->d_taken,
-                                                                          p->d_current);
+    schedule_advance_kernel<<<dim3(1), dim3(64), 0, (hipStream_t)stream>>>(p->d_header);
     RLX_HIP(hipGetLastError());
     return RLX_OK;
 }
@@ -1799,11 +2060,22 @@ int rlx_plan_schedule_position(rlx_plan* p, int64_t* steps_taken, int64_t* n_ste
     if (!plan_ok(p) || !p->d_sched) return RLX_ERR_INVALID_ARG;
     const int ready = plan_launchable(p);
     if (ready != RLX_OK) return ready;
-    int64_t taken = 0;
+    SchedHeader h;
     RLX_HIP(hipStreamSynchronize((hipStream_t)stream));
-    RLX_HIP(hipMemcpy(&taken, p->d_taken, sizeof(taken), hipMemcpyDeviceToHost));
-    if (steps_taken) *steps_taken = taken;
-    if (n_steps) *n_steps = p->sched_len;
+    RLX_HIP(hipMemcpy(&h, p->d_header, sizeof(h), hipMemcpyDeviceToHost));
+    if (steps_taken) *steps_taken = h.taken;
+    if (n_steps) *n_steps = h.len;
+    return RLX_OK;
+}
+
+int rlx_plan_schedule_overrun(rlx_plan* p, int64_t* overrun, void* stream) {
+    if (!plan_ok(p) || !p->d_sched || !overrun) return RLX_ERR_INVALID_ARG;
+    const int ready = plan_launchable(p);
+    if (ready != RLX_OK) return ready;
+    SchedHeader h;
+    RLX_HIP(hipStreamSynchronize((hipStream_t)stream));
+    RLX_HIP(hipMemcpy(&h, p->d_header, sizeof(h), hipMemcpyDeviceToHost));
+    *overrun = h.overrun;
     return RLX_OK;
 }
 
@@ -1826,6 +2098,10 @@ int rlx_set_tuning(const char* key, int64_t value) {
         if (value != 0 && value != 8 && value != 16 && value != 32 && value != 40) return RLX_ERR_INVALID_ARG;
         g_tuning.final_batch = value;
     }
+    else if (!strcmp(key, "norm_fused")) {
+        if (value > 2) return RLX_ERR_INVALID_ARG;
+        g_tuning.norm_fused = value;
+    }
     else if (!strcmp(key, "convert_variant")) {
         if (value >= kNumConvertVariants) return RLX_ERR_INVALID_ARG;
         g_tuning.convert_variant = value;
@@ -1841,6 +2117,7 @@ int64_t rlx_get_tuning(const char* key) {
     if (!strcmp(key, "norm_pack")) return g_tuning.norm_pack;
     if (!strcmp(key, "convert_variant")) return g_tuning.convert_variant;
     if (!strcmp(key, "final_batch")) return g_tuning.final_batch;
+    if (!strcmp(key, "norm_fused")) return g_tuning.norm_fused;
     return -1;
 }
 

@@ -176,6 +176,7 @@ class AdamWOptimizer:
         self.lr, self.beta1, self.beta2, self.eps, self.weight_decay = lr, beta1, beta2, eps, weight_decay
         self.store = store
         self.step_ = 0
+        self._scheduled_lrs, self._scheduled_from = [], 0       # the uploaded step table and get_step() at its upload
         self.plan = B.Plan(store.descs(extra_grad_only), chunk_elems)
 
     def set_lr(self, new_lr):
@@ -210,13 +211,34 @@ class AdamWOptimizer:
 
     def step_scheduled(self, fused_clip=False, zero_grads=False, stream=None):
         """step() with the hyper-parameters of the uploaded table; the device moves on to the next entry by
-        itself, so a captured launch can be replayed without any host write in between."""
-        k = self.step_ - self._scheduled_from
-        if 0 <= k < len(self._scheduled_lrs):
+        itself, so a recorded launch can be replayed without any host write in between, through this window and
+        every later upload (the recorded launch does not depend on the table's address or length).
+        A call while torch's current stream is being captured records the launch and does not count as a step
+        (count the replays with note_replayed_steps); an eager call counts, and raises if the table is used up
+        or none was uploaded, instead of running with the last entry's learning rate and bias corrections."""
+        import torch
+        st = _stream() if stream is None else stream
+        if not torch.cuda.is_current_stream_capturing():
+            k = self.step_ - self._scheduled_from
+            if not 0 <= k < len(self._scheduled_lrs):
+                raise RuntimeError("step_scheduled: the uploaded table of %d steps is used up (or none was uploaded); "
+                                   "call upload_schedule for the next window first" % len(self._scheduled_lrs))
             self.lr = self._scheduled_lrs[k]           # host-side bookkeeping only; the device reads its table
-        self.step_ += 1
+            self.step_ += 1
         flags = (B.CLIP_FUSED if fused_clip else 0) | (B.STEP_ZERO_GRADS if zero_grads else 0)
-        self.plan.adamw_scheduled(flags, _stream() if stream is None else stream)
+        self.plan.adamw_scheduled(flags, st)
+
+    def note_replayed_steps(self, n):
+        """After n replays of a recorded step_scheduled: get_step() += n.  Raises if that was more than the
+        uploaded table held (the excess reused the table's last entry)."""
+        self.step_ += n
+        k = self.step_ - self._scheduled_from
+        if 0 < k <= len(self._scheduled_lrs):
+            self.lr = self._scheduled_lrs[k - 1]
+        if k > len(self._scheduled_lrs):
+            raise RuntimeError("%d scheduled steps have run since a table of %d was uploaded: the last %d reused the "
+                               "table's last learning rate and bias corrections"
+                               % (k, len(self._scheduled_lrs), k - len(self._scheduled_lrs)))
 
     # --- optimizer state on disk (the reference's save_checkpoint is a stub, trainer.h:317-319) ----
     # One format, shared with the C++ AdamWOptimizer (rl.cu_amd/host/training/optimizer.h): "RLXOPT02", int32

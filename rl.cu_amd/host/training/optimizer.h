@@ -209,6 +209,7 @@ public:
         if (frozen != embed_frozen_) {
             embed_frozen_ = frozen;
             if (plan_) { RLX_CHECK(rlx_plan_destroy(plan_)); plan_ = nullptr; }
+            sched_len_ = 0;
         }
     }
 
@@ -247,8 +248,23 @@ public:
     // Steps without the host (a recorded norm + update replayed step after step).  upload_schedule puts the
     // hyper-parameters of the next n steps (steps get_step()+1, ...) on the device: the given learning rates and
     // the bias corrections formed here with powf, as in step().  step_scheduled launches the update with the
-    // current entry; the device then moves on to the next entry by itself, so a captured step_scheduled can be
-    // replayed with nothing written by the host in between (advance get_step() with note_replayed_steps).
+    // current entry; the device then moves on to the next entry by itself, so a recorded step_scheduled can be
+    // replayed with nothing written by the host in between, through this window and every later one (the
+    // recorded launch does not depend on the table's address or length).
+    //
+    //     optimizer.set_fused_clip(true);
+    //     optimizer.upload_schedule(grads, lrs, n);              // window 1
+    //     hipStreamBeginCapture(s, ...);
+    //     optimizer.clip_grad_norm_async(grads, max_norm, s);    // norm and clip scale, nothing read by the host
+    //     optimizer.step_scheduled(grads, s);                    // recorded, not run: get_step() does not move
+    //     hipStreamEndCapture(s, &graph); ...
+    //     for (k = 0; k < n; k++) hipGraphLaunch(exec, s);       // new gradients before each replay
+    //     optimizer.note_replayed_steps(n);                      // get_step() += n
+    //     optimizer.upload_schedule(grads, next_lrs, n2);        // window 2: same graph, replay on
+    //
+    // A call while `stream` is being captured does not count as a step; every eager call does.  Running more
+    // scheduled steps than the table holds would reuse the last entry's learning rate and bias corrections: an
+    // eager step_scheduled refuses (exits with a message), note_replayed_steps reports it.
     // The table belongs to the plan: if the gradient pools move or set_embed_frozen changes, the plan is rebuilt
     // and the schedule has to be uploaded again.
     template <class Grads>
@@ -261,16 +277,55 @@ public:
             sp.bias_correction2 = 1.0f - powf(beta2, (float)(step_ + 1 + k));
         }
         RLX_CHECK(rlx_plan_schedule_upload(plan_for(grads), steps.data(), n, (void*)stream));
+        sched_from_ = step_;
+        sched_len_ = n;
+    }
+
+    // fused_clip: apply, inside the update, the clip scale that the last norm of plan_for(grads) left on the
+    // device.  The two-argument form takes it from clip_grad_norm_ / clip_grad_norm_async having run with
+    // set_fused_clip(true) since the last step.
+    template <class Grads>
+    void step_scheduled(Grads* grads, hipStream_t stream, bool fused_clip) {
+        rlx_plan* plan = plan_for(grads);
+        hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+        if (stream) HIP_CHECK(hipStreamIsCapturing(stream, &capturing));
+        if (capturing == hipStreamCaptureStatusNone) {
+            if (step_ - sched_from_ >= sched_len_) {
+                fprintf(stderr, "[AdamW] step_scheduled: the uploaded table of %d steps is used up (or none was uploaded "
+                                "for these gradient pools); call upload_schedule for the next window first\n", sched_len_);
+                exit(1);
+            }
+            step_++;
+        }
+        const int flags = (fused_clip ? RLX_CLIP_FUSED : 0) | (zero_grads_ ? RLX_STEP_ZERO_GRADS : 0);
+        RLX_CHECK(rlx_plan_adamw_scheduled(plan, flags, (void*)stream));
     }
     template <class Grads>
     void step_scheduled(Grads* grads, hipStream_t stream = 0) {
         const bool fused = clip_pending_;
         clip_pending_ = false;
-        step_++;
-        const int flags = (fused ? RLX_CLIP_FUSED : 0) | (zero_grads_ ? RLX_STEP_ZERO_GRADS : 0);
-        RLX_CHECK(rlx_plan_adamw_scheduled(plan_for(grads), flags, (void*)stream));
+        step_scheduled(grads, stream, fused);
     }
-    void note_replayed_steps(int n) { step_ += n; }
+    // After n replays of a recorded step_scheduled.  Returns false (and says so) if that was more than the table held.
+    bool note_replayed_steps(int n) {
+        step_ += n;
+        if (step_ - sched_from_ <= sched_len_) return true;
+        fprintf(stderr, "[AdamW] %d scheduled steps have run since a table of %d was uploaded: the last %d reused the "
+                        "table's last learning rate and bias corrections\n", step_ - sched_from_, sched_len_,
+                step_ - sched_from_ - sched_len_);
+        return false;
+    }
+
+    // The half of clip_grad_norm_ that needs no host (so that it can be recorded): norm and clip scale stay on
+    // the device.  With set_fused_clip(true) the next step / step_scheduled applies the scale; otherwise the
+    // scale pass is launched here (it reads the scale on the device and touches nothing when it is 1).
+    template <class Grads>
+    void clip_grad_norm_async(Grads* grads, float max_norm, hipStream_t stream = 0) {
+        rlx_plan* plan = plan_for(grads);
+        RLX_CHECK(rlx_plan_grad_norm(plan, max_norm, (void*)stream));
+        if (fused_clip_) clip_pending_ = true;
+        else RLX_CHECK(rlx_plan_scale_grads(plan, (void*)stream));
+    }
 
     // Trainer::clip_grad_norm_ (trainer.h:323-352) over the same gradient type: clips all gradients
     // (half_pool + float_pool) so that the global L2 norm is <= max_norm and returns the pre-clip norm
@@ -412,6 +467,7 @@ public:
             grads->float_pool_bytes == plan_float_bytes_)
             return plan_;
         if (plan_) { RLX_CHECK(rlx_plan_destroy(plan_)); plan_ = nullptr; }
+        sched_len_ = 0;                 // an uploaded step table went with the old plan
         assert(grads->half_pool_bytes / sizeof(half) == n16_);
         assert(grads->float_pool_bytes / sizeof(float) >= n32_);
         rlx_tensor_desc d[4];
@@ -458,6 +514,7 @@ private:
     bool embed_frozen_ = false;
     bool fused_clip_ = false, zero_grads_ = false;
     bool clip_pending_ = false;     // a fused clip_grad_norm_() has run since the last step()
+    int sched_from_ = 0, sched_len_ = 0;   // get_step() at the last upload_schedule and that table's length
 
     size_t fp16_offset(int layer, int proj) const {
         assert(pools_.num_layers > 0 && layer >= 0 && layer < pools_.num_layers && proj >= 0 && proj < 7);
@@ -537,6 +594,7 @@ private:
         plan_ = o.plan_; plan_half_ = o.plan_half_; plan_float_ = o.plan_float_; plan_float_bytes_ = o.plan_float_bytes_;
         embed_frozen_ = o.embed_frozen_; stage_limit_ = o.stage_limit_;
         fused_clip_ = o.fused_clip_; zero_grads_ = o.zero_grads_; clip_pending_ = o.clip_pending_;
+        sched_from_ = o.sched_from_; sched_len_ = o.sched_len_;
         o.plan_ = nullptr; o.fp16_state_ = nullptr; o.fp32_state_ = nullptr;
         o.fp16_master_ = o.fp16_m_ = o.fp16_v_ = o.fp32_m_ = o.fp32_v_ = nullptr;
     }

@@ -12,6 +12,7 @@
 //   7. frozen embedding flagged in the plan, gradients cleared inside the update
 //   8. optimizer state save / load   9. train loop with LR schedule and JSON-lines log
 //   10. gradient pools   11. training_step with accumulation   12. steps from an uploaded table of hyper-parameters
+//   13. one recorded clip + scheduled step replayed through three uploaded windows, against the oracle
 // The oracle (liborc_adamw.so) is used as the checker only.
 #include <cmath>
 #include <cstdint>
@@ -33,6 +34,14 @@ void orc_adamw_fp32(float*, const float*, float*, float*, int64_t, float, float,
 float orc_clip_grad_norm(uint16_t*, int64_t, float*, int64_t, float, float*);
 double orc_sum_sq_half(const uint16_t*, int64_t);
 double orc_sum_sq_float(const float*, int64_t);
+int64_t orc_sumsq_mirror_partials(const void* g, int is_f32, int64_t n, int chunk, double* partials);
+double orc_sumsq_mirror_total(const double* partials, int64_t n_partials, int chunk);
+float orc_clip_scale(float sum_sq, float max_norm, float* norm);
+void orc_scale_half(uint16_t*, float, int64_t);
+void orc_scale_float(float*, float, int64_t);
+void orc_optimizer_step(float* master, uint16_t* pool16, const uint16_t* g16, float* m16, float* v16, int64_t n16,
+                        int64_t proj_n, float* pool32, const float* g32, float* m32, float* v32, int64_t n32, float lr,
+                        float beta1, float beta2, float eps, float wd, int* step);
 }
 
 static int g_fails = 0;
@@ -82,6 +91,60 @@ template <typename T> static std::vector<T> d2h(const T* d, size_t n) {
     HIP_CHECK(hipMemcpy(h.data(), d, n * sizeof(T), hipMemcpyDeviceToHost));
     return h;
 }
+
+// The oracle's copy of a Fixture's training state, advanced on the host in the reference's order
+// (trainer.h:279-286): norm of all gradients, added up in the device's fixed order so that it can be compared
+// bit for bit, clip rule, scale pass if norm > max, optimizer step with the three decay groups.
+struct OracleReplay {
+    Fixture& f;
+    std::vector<float> master, m16, v16, w32, m32, v32;
+    std::vector<uint16_t> w16;
+    int step = 0;
+    float beta1 = 0.9f, beta2 = 0.999f, eps = 1e-8f, wd = 0.01f;
+
+    explicit OracleReplay(Fixture& fx) : f(fx), master(fx.n16), m16(fx.n16, 0.0f), v16(fx.n16, 0.0f), w32(fx.h_w32),
+                                         m32(fx.n32, 0.0f), v32(fx.n32, 0.0f), w16(fx.h_w16) {
+        for (size_t i = 0; i < fx.n16; i++) master[i] = orc_h2f(fx.h_w16[i]);
+    }
+    // One step on the gradients that the device holds now.  Returns the pre-clip norm.
+    float advance(float lr, float max_norm, int64_t chunk) {
+        std::vector<uint16_t> g16 = d2h((const uint16_t*)f.g16, f.n16);
+        std::vector<float> g32 = d2h((const float*)f.g32, f.n32 + f.tail);
+        float norm = 0.0f;
+        if (max_norm > 0.0f) {
+            std::vector<double> partials((f.n16 + f.n32 + f.tail) / 512 + 16);
+            int64_t k = 0;      // plan order: projections, embedding, norm gradients, workspace tail
+            k += orc_sumsq_mirror_partials(g16.data(), 0, (int64_t)f.proj_n, (int)chunk, partials.data() + k);
+            k += orc_sumsq_mirror_partials(g16.data() + f.proj_n, 0, (int64_t)f.embed_n, (int)chunk, partials.data() + k);
+            k += orc_sumsq_mirror_partials(g32.data(), 1, (int64_t)f.n32, (int)chunk, partials.data() + k);
+            k += orc_sumsq_mirror_partials(g32.data() + f.n32, 1, (int64_t)f.tail, (int)chunk, partials.data() + k);
+            const float scale = orc_clip_scale((float)orc_sumsq_mirror_total(partials.data(), k, (int)chunk), max_norm, &norm);
+            if (norm > max_norm) {
+                orc_scale_half(g16.data(), scale, (int64_t)f.n16);
+                orc_scale_float(g32.data(), scale, (int64_t)(f.n32 + f.tail));
+            }
+        }
+        orc_optimizer_step(master.data(), w16.data(), g16.data(), m16.data(), v16.data(), (int64_t)f.n16,
+                           (int64_t)f.proj_n, w32.data(), g32.data(), m32.data(), v32.data(), (int64_t)f.n32, lr, beta1,
+                           beta2, eps, wd, &step);
+        return norm;
+    }
+    // Values of the device state (weights, master copy, moments) that differ from the oracle's in any bit.
+    size_t differences(AdamWOptimizer& opt) const {
+        size_t diff = 0;
+        const auto dw16 = d2h((const uint16_t*)f.w16, f.n16);
+        const auto dw32 = d2h((const float*)f.w32, f.n32);
+        const auto dmaster = d2h((const float*)opt.fp16_master(), f.n16);
+        const auto dm16 = d2h((const float*)opt.fp16_m(), f.n16), dv16 = d2h((const float*)opt.fp16_v(), f.n16);
+        const auto dm32 = d2h((const float*)opt.fp32_m(), f.n32), dv32 = d2h((const float*)opt.fp32_v(), f.n32);
+        for (size_t i = 0; i < f.n16; i++)
+            diff += dw16[i] != w16[i] || memcmp(&dmaster[i], &master[i], 4) || memcmp(&dm16[i], &m16[i], 4) ||
+                    memcmp(&dv16[i], &v16[i], 4);
+        for (size_t i = 0; i < f.n32; i++)
+            diff += memcmp(&dw32[i], &w32[i], 4) || memcmp(&dm32[i], &m32[i], 4) || memcmp(&dv32[i], &v32[i], 4);
+        return diff;
+    }
+};
 
 // 1. FP32 path vs the CPU loop of the reference's test (step 1, division by the bias corrections)
 static void test_cpu_reference_fp32() {
@@ -312,29 +375,68 @@ static void test_checkpoint() {
     if (ok && diff == 0 && refused && ob.get_step() == 5) PASS(name); else FAIL(name, "ok=%d diff=%zu refused=%d", ok, diff, refused);
 }
 
-// 9. scheduled learning rate, train loop, JSON-lines log
+// 9. scheduled learning rate, train loop, JSON-lines log: the loop's logged pre-clip norm (trainer.h:208-216,
+//    288, 351) and the state it leaves are those of the oracle replaying set_lr -> clip -> step on the host;
+//    the state file written at save_steps holds the oracle's state of that step
 static void test_train_loop() {
-    const char* name = "train loop with LR schedule and JSONL log";
+    const char* name = "train loop with LR schedule and JSONL log == oracle replay";
     const std::string dir = "/tmp/rlx_test_run";
     std::filesystem::remove_all(dir);
+    std::filesystem::create_directories(dir);
     Fixture f(5e-3f);
     AdamWOptimizer opt(f.pools, 1e-3f);
+    OracleReplay oracle(f);
     LRScheduler sched;
     sched.init_cosine(1e-3f, 1e-4f, 2, 8);
     OptimStepConfig c; c.max_grad_norm = 0.25f; c.fused_clip = true;
     OptimStep tail(&opt, c);
     TrainLoopConfig lc; lc.total_steps = 8; lc.logging_steps = 2; lc.tokens_per_step = 4096.0f;
+    lc.save_steps = 4; lc.save_path = dir + "/opt_state.bin";
+    const int64_t chunk = rlx_plan_chunk_elems(opt.plan_for(&f.grads));
+    std::vector<float> norms;                       // the oracle's pre-clip norm of every step
+    size_t saved_diff = 0;
     int steps;
     {
         Logger logger(dir);
         steps = run_train_loop(opt, sched, logger, tail, &f.grads, [&](int s) {
+            if (s == 4) {     // the loop has just written the state of step 4: load it into a second optimizer
+                Fixture g(5e-3f);
+                AdamWOptimizer reloaded(g.pools, 1e-3f);
+                OracleReplay then = oracle;
+                const bool ok = reloaded.load_state(lc.save_path) && reloaded.get_step() == 4;
+                // weights are not part of the state file: compare master copy and moments
+                const auto dmaster = d2h((const float*)reloaded.fp16_master(), g.n16);
+                const auto dm = d2h((const float*)reloaded.fp16_m(), g.n16), dv = d2h((const float*)reloaded.fp16_v(), g.n16);
+                const auto dm32 = d2h((const float*)reloaded.fp32_m(), g.n32), dv32 = d2h((const float*)reloaded.fp32_v(), g.n32);
+                saved_diff += ok ? 0 : 1;
+                for (size_t i = 0; i < g.n16; i++)
+                    saved_diff += memcmp(&dmaster[i], &then.master[i], 4) || memcmp(&dm[i], &then.m16[i], 4) ||
+                                  memcmp(&dv[i], &then.v16[i], 4);
+                for (size_t i = 0; i < g.n32; i++) saved_diff += memcmp(&dm32[i], &then.m32[i], 4) || memcmp(&dv32[i], &then.v32[i], 4);
+            }
             RLX_CHECK(rlx_fill_f16((uint16_t*)f.g16, f.n16, 100 + s, 0, 0.0f, 5e-3f, 0, 0, 0, nullptr));
+            HIP_CHECK(hipDeviceSynchronize());
+            norms.push_back(oracle.advance(sched.get_lr(s), c.max_grad_norm, chunk));
             return 3.0f / (1 + s);
         }, lc);
         bool ok = steps == 8 && opt.get_step() == 8 && logger.history().size() == 4 && opt.lr == sched.get_lr(7) &&
                   logger.history()[0].step == 2 && fabsf(logger.last("loss") - (3.0f / 7 + 3.0f / 8) / 2) < 1e-6f &&
-                  logger.last("grad_norm") > 0.25f && std::isnan(logger.last("nope"));
-        if (!ok) { FAIL(name, "loop state"); return; }
+                  std::isnan(logger.last("nope"));
+        // every logged window mean of grad_norm is the FP32 mean of the oracle's norms of its two steps
+        size_t norm_diff = 0;
+        for (size_t w = 0; ok && w < 4; w++) {
+            const float want = (0.0f + norms[2 * w] + norms[2 * w + 1]) / 2.0f;
+            const float got = logger.history()[w].values.at("grad_norm");
+            norm_diff += memcmp(&want, &got, 4) != 0;
+            ok = ok && norms[2 * w] > 0.25f && fabsf(got - want) <= 1e-7f * want;
+        }
+        const size_t state_diff = oracle.differences(opt);
+        printf("  logged grad_norm windows differing from the oracle's: %zu; state values differing after 8 steps: %zu; "
+               "in the state file of step 4: %zu\n", norm_diff, state_diff, saved_diff);
+        if (!ok || norm_diff || state_diff || saved_diff || oracle.step != 8) {
+            FAIL(name, "ok=%d norm_diff=%zu state_diff=%zu saved_diff=%zu", ok, norm_diff, state_diff, saved_diff);
+            return;
+        }
     }
     FILE* fp = fopen((dir + "/train_log.jsonl").c_str(), "r");
     int lines = 0; char buf[1024]; bool shape = fp != nullptr;
@@ -488,6 +590,69 @@ static void test_scheduled_steps() {
     else FAIL(name, "ok=%d diff=%zu taken=%lld total=%lld refused=%d", ok, diff, (long long)taken, (long long)total, refused);
 }
 
+// 13. The recorded step of the header's recipe: clip_grad_norm_async + step_scheduled captured once into a HIP
+//     graph after the first upload, replayed through window 1 (3 steps), a longer window 2 (6 steps) and a shorter
+//     window 3 (2 steps).  The reference sets the scheduler's rate before every step of the whole run
+//     (trainer.h:193-194) and forms the bias corrections from the step number (optimizer.h:120-122): the oracle
+//     replays exactly that on the host, and weights, master copy and moments must agree bit for bit after every
+//     window; get_step() counts the replays and not the capture; no step overruns its table.
+static void test_recorded_step_across_windows() {
+    const char* name = "one recorded clip + scheduled step through three uploaded windows == oracle";
+    Fixture f(5e-3f);
+    AdamWOptimizer opt(f.pools, 1e-3f);
+    OracleReplay oracle(f);
+    LRScheduler sched;
+    sched.init_cosine(1e-3f, 1e-5f, 2, 11);
+    const float max_norm = 0.25f;
+    opt.set_fused_clip(true);
+    hipStream_t s;
+    HIP_CHECK(hipStreamCreate(&s));
+    const int64_t chunk = rlx_plan_chunk_elems(opt.plan_for(&f.grads));
+    const int windows[3] = {3, 6, 2};
+    hipGraph_t graph = nullptr;
+    hipGraphExec_t exec = nullptr;
+    bool ok = true;
+    size_t diff = 0;
+    int global = 0;
+    for (int w = 0; w < 3; w++) {
+        const int n = windows[w];
+        std::vector<float> lrs((size_t)n);
+        for (int k = 0; k < n; k++) lrs[(size_t)k] = sched.get_lr(global + k);
+        ok = ok && opt.get_step() == global;
+        opt.upload_schedule(&f.grads, lrs.data(), n, s);
+        if (!exec) {
+            HIP_CHECK(hipStreamBeginCapture(s, hipStreamCaptureModeThreadLocal));
+            opt.clip_grad_norm_async(&f.grads, max_norm, s);
+            opt.step_scheduled(&f.grads, s);
+            HIP_CHECK(hipStreamEndCapture(s, &graph));
+            HIP_CHECK(hipGraphInstantiate(&exec, graph, nullptr, nullptr, 0));
+            ok = ok && opt.get_step() == 0;               // recording is not a step
+        }
+        for (int k = 0; k < n; k++) {
+            RLX_CHECK(rlx_fill_f16((uint16_t*)f.g16, f.n16, 300 + global + k, 0, 0.0f, 2e-3f * (float)(global + k + 1), 0, 0, 0, s));
+            RLX_CHECK(rlx_fill_f32(f.g32, f.n32 + f.tail, 400 + global + k, 0, 0.0f, 3e-3f, 0, 0, 0, s));
+            HIP_CHECK(hipStreamSynchronize(s));
+            const float want = oracle.advance(lrs[(size_t)k], max_norm, chunk);
+            HIP_CHECK(hipGraphLaunch(exec, s));
+            HIP_CHECK(hipStreamSynchronize(s));
+            float got = 0.0f;
+            RLX_CHECK(rlx_plan_norm_read(opt.plan_for(&f.grads), &got, nullptr, nullptr, s));
+            int64_t taken = -1, total = -1, overrun = -1;
+            RLX_CHECK(rlx_plan_schedule_position(opt.plan_for(&f.grads), &taken, &total, s));
+            RLX_CHECK(rlx_plan_schedule_overrun(opt.plan_for(&f.grads), &overrun, s));
+            ok = ok && memcmp(&got, &want, 4) == 0 && want > max_norm && taken == k + 1 && total == n && overrun == 0;
+        }
+        ok = ok && opt.note_replayed_steps(n);
+        global += n;
+        diff += oracle.differences(opt);
+    }
+    ok = ok && opt.get_step() == 11 && oracle.step == 11;
+    HIP_CHECK(hipGraphExecDestroy(exec));
+    HIP_CHECK(hipGraphDestroy(graph));
+    HIP_CHECK(hipStreamDestroy(s));
+    if (ok && diff == 0) PASS(name); else FAIL(name, "ok=%d diff=%zu step=%d", ok, diff, opt.get_step());
+}
+
 int main() {
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev == 0) {
@@ -507,6 +672,7 @@ int main() {
     test_grad_pools();
     test_accumulation();
     test_scheduled_steps();
+    test_recorded_step_across_windows();
     printf("=== %s (%d failure%s) ===\n", g_fails ? "FAILED" : "ALL PASSED", g_fails, g_fails == 1 ? "" : "s");
     return g_fails;
 }

@@ -32,7 +32,7 @@ float orc_clip_scale(float sum_sq, float max_norm, float* norm_out);
 double orc_sum_sq_half(const uint16_t*, int64_t);
 double orc_sum_sq_float(const float*, int64_t);
 int64_t orc_sumsq_mirror_partials(const void* g, int is_f32, int64_t n, int chunk, double* partials);
-double orc_sumsq_mirror_final(const double* partials, int64_t n_partials);
+double orc_sumsq_mirror_total(const double* partials, int64_t n_partials, int chunk);
 void orc_optimizer_step(float* fp16_master, uint16_t* fp16_pool, const uint16_t* half_grads, float* fp16_m, float* fp16_v,
                         int64_t n16, int64_t proj_n, float* fp32_pool, const float* float_grads, float* fp32_m,
                         float* fp32_v, int64_t n32, float lr, float beta1, float beta2, float eps, float weight_decay,
@@ -246,7 +246,7 @@ static Expected oracle_tail(World& w, const TrainingConfig& cfg, float lr, int64
         k += orc_sumsq_mirror_partials(e.g16.data() + w.proj_n, 0, (int64_t)w.embed_n, (int)chunk, partials.data() + k);
         k += orc_sumsq_mirror_partials(e.g32.data(), 1, (int64_t)w.n32, (int)chunk, partials.data() + k);
         k += orc_sumsq_mirror_partials(e.g32.data() + w.n32, 1, (int64_t)w.tail, (int)chunk, partials.data() + k);
-        const double sum_sq = orc_sumsq_mirror_final(partials.data(), k);
+        const double sum_sq = orc_sumsq_mirror_total(partials.data(), k, (int)chunk);
         const float scale = orc_clip_scale((float)sum_sq, cfg.max_grad_norm, &e.norm);
         const double exact = sqrt(orc_sum_sq_half(e.g16.data(), (int64_t)w.n16) +
                                   orc_sum_sq_float(e.g32.data(), (int64_t)(w.n32 + w.tail)));

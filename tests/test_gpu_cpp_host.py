@@ -1,5 +1,7 @@
 """Runs the C++ host-side test (the reference-shaped AdamWOptimizer / clip_grad_norm_ / launch_adamw_*
-mirror in rl.cu_amd/host) on the GPU.  The binary is built beforehand by __graft_entry__.build()."""
+mirror in rl.cu_amd/host) on the GPU.  The binaries are built beforehand by __graft_entry__.build(); make runs
+again here every time, so that a binary older than the headers it was built from is never what gets tested (an
+up-to-date one costs nothing)."""
 import os
 import subprocess
 
@@ -12,13 +14,12 @@ EXE = os.path.join(ROOT, "tests", "cpp", "test_adamw_host.bin")
 
 
 def test_cpp_host_mirror(torch_gpu):
-    if not os.path.exists(EXE):
-        subprocess.run(["make", "-C", os.path.dirname(EXE), "-s"], check=True)
+    subprocess.run(["make", "-C", os.path.dirname(EXE), "-s"], check=True)
     res = subprocess.run([EXE], capture_output=True, text=True, timeout=100)
     print(res.stdout)
     print(res.stderr)
     assert res.returncode == 0, res.stdout + res.stderr
-    assert res.stdout.count("[PASS]") == 12 and "[FAIL]" not in res.stdout
+    assert res.stdout.count("[PASS]") == 13 and "[FAIL]" not in res.stdout
 
 
 def test_reference_call_sites_compile_unchanged_and_match_the_oracle(torch_gpu):
@@ -26,8 +27,7 @@ def test_reference_call_sites_compile_unchanged_and_match_the_oracle(torch_gpu):
     path reads, the lines of the reference's trainer.h:280-286 and GRPO_trainer.h:508-514 unchanged, every result
     bit-identical to the oracle replaying the reference's order of operations."""
     exe = os.path.join(ROOT, "tests", "cpp", "test_reference_callsites.bin")
-    if not os.path.exists(exe):
-        subprocess.run(["make", "-C", os.path.dirname(exe), "-s"], check=True)
+    subprocess.run(["make", "-C", os.path.dirname(exe), "-s"], check=True)
     res = subprocess.run([exe], capture_output=True, text=True, timeout=200)
     print(res.stdout)
     print(res.stderr)

@@ -161,8 +161,7 @@ class OracleReplay:
 
 def run_tool(*args):
     import subprocess
-    if not os.path.exists(XTOOL):
-        subprocess.run(["make", "-C", os.path.dirname(XTOOL), "-s"], check=True)
+    subprocess.run(["make", "-C", os.path.dirname(XTOOL), "-s"], check=True)      # up to date: costs nothing
     return subprocess.run([XTOOL] + [str(a) for a in args], capture_output=True, text=True, timeout=100)
 
 
@@ -236,25 +235,52 @@ def test_state_saved_by_python_loads_in_cxx_and_continues_as_the_oracle(O, B, L,
         assert run_tool("load", tmp_path, 3, 1).returncode == 3
 
 
-def test_train_loop_logs_jsonl(L, host, torch_gpu, tmp_path, capsys):
+def test_train_loop_logs_jsonl(O, L, host, torch_gpu, tmp_path, capsys):
     """Cosine schedule with warm-up drives set_lr; every second step one JSON line with the window means of
-    loss, lr, grad_norm, step_ms, tok_per_sec (the keys of include/training/trainer.h:208-212)."""
+    loss, lr, grad_norm, step_ms, tok_per_sec (the keys of include/training/trainer.h:208-212).
+    The loop is pinned to the oracle: the reference logs the pre-clip norm that clip_grad_norm_ returns and its
+    weights follow from set_lr + clip + step (trainer.h:183-225, 288, 351), so the oracle replays the eight steps
+    on the host (scheduler's rate -> norm in the plan's order -> clip rule -> step) and every logged window mean
+    of grad_norm, the state file written at save_steps and the parameters and moments after the loop must be
+    the oracle's, bit for bit."""
+    import numpy as np
+    from test_gpu_plan import compare, host_copy, oracle_step
+    from util import HYPER, bits
+    torch = torch_gpu
     specs, st, opt = make(L, host, False)
     sched = host.LRScheduler()
     sched.init_cosine(1e-3, 1e-4, 2, 8)
     log_dir = str(tmp_path / "run")
     logger = host.Logger(log_dir)
-    losses = []
+    losses, oracle_norms = [], []
+    torch.cuda.synchronize()
+    hs = host_copy(st)
+    state_path = str(tmp_path / "opt.state")
 
     def produce(step):
+        if step == 4:       # the loop has just saved the state of step 4: it reloads to the oracle's state
+            _, st_b, opt_b = make(L, host, False)
+            opt_b.load_state(state_path)
+            assert opt_b.get_step() == 4 and opt_b.lr == sched.get_lr(3)
+            for i, h in enumerate(hs):
+                assert np.array_equal(bits(st_b.state(i, "m")), h["m"]) and np.array_equal(bits(st_b.state(i, "v")), h["v"])
         st.fill("g", 100 + step, 0.0, 5e-3)
+        torch.cuda.synchronize()
+        for i, h in enumerate(hs):
+            h["g"] = bits(st.grad(i))
+        ssq, _ = O.sumsq_mirror([h["g"] for h in hs], opt.plan.chunk_elems)
+        scale, norm = O.clip_scale(np.float32(ssq), 0.5)
+        oracle_step(O, L, specs, hs, step + 1, dict(HYPER, lr=sched.get_lr(step)), clip_scale=scale)
+        oracle_norms.append(np.float32(norm))
         losses.append(3.0 / (1 + step))
         return losses[-1]
 
     done = host.train_loop(opt, sched, logger, produce, total_steps=8, max_grad_norm=0.5, logging_steps=2,
-                           save_steps=4, save_path=str(tmp_path / "opt.state"), tokens_per_step=4096)
+                           save_steps=4, save_path=state_path, tokens_per_step=4096)
     logger.close()
-    assert done == 8 and opt.get_step() == 8 and os.path.exists(str(tmp_path / "opt.state"))
+    assert done == 8 and opt.get_step() == 8 and os.path.exists(state_path)
+    torch.cuda.synchronize()
+    assert compare(st, hs, "after the loop") == 0
     rows = [json.loads(l) for l in open(os.path.join(log_dir, "train_log.jsonl"))]
     assert [r["step"] for r in rows] == [2, 4, 6, 8]
     assert all(sorted(r) == ["grad_norm", "loss", "lr", "step", "step_ms", "tok_per_sec"] for r in rows)
@@ -262,7 +288,9 @@ def test_train_loop_logs_jsonl(L, host, torch_gpu, tmp_path, capsys):
         s0, s1 = 2 * k, 2 * k + 1
         assert abs(r["loss"] - (losses[s0] + losses[s1]) / 2) < 1e-6
         assert abs(r["lr"] - (sched.get_lr(s0) + sched.get_lr(s1)) / 2) < 1e-9
-        assert r["grad_norm"] > 0.5 and r["step_ms"] > 0 and r["tok_per_sec"] > 0
+        want = np.float32(np.float32(np.float32(0.0) + oracle_norms[s0]) + oracle_norms[s1]) / np.float32(2)   # FP32 window mean
+        assert abs(r["grad_norm"] - float(want)) <= 1e-7 * float(want) and r["grad_norm"] == float(want)
+        assert oracle_norms[s0] > 0.5 and r["step_ms"] > 0 and r["tok_per_sec"] > 0
     assert abs(opt.lr - sched.get_lr(7)) < 1e-12
     assert logger.last("loss") == rows[-1]["loss"] and math.isnan(logger.last("nope")) and len(logger.history()) == 4
     assert "[step 8]" in capsys.readouterr().out

@@ -448,7 +448,8 @@ def test_scheduled_steps_replay_without_the_host(O, L, host, B, torch_gpu):
     decaying learning rate, host-computed bias corrections) are uploaded once, and the graph is replayed five
     times with NO host write of hyper-parameters in between: only new gradients arrive (eager fills and
     synchronisations between the replays).  Every replay equals the oracle; the sixth, eager, scheduled step
-    uses the sixth entry; a seventh reuses it (the table is exhausted) and the position saturates."""
+    uses the sixth entry; the host mirror refuses a seventh; launched through the C ABI all the same, it reuses
+    the last entry (the table is exhausted), the position saturates and the overrun is counted."""
     torch = torch_gpu
     specs = L.qwen3_tensor_list(MINI, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
     st = host.ParamStore(specs)
@@ -494,15 +495,23 @@ def test_scheduled_steps_replay_without_the_host(O, L, host, B, torch_gpu):
         check(step, lrs[step - 1])
         assert opt.plan.schedule_position() == (step, 6)
     # eager scheduled steps continue where the replays left off
-    opt.step_ = 5
+    assert opt.get_step() == 0                                   # recording counted nothing
+    opt.note_replayed_steps(5)
+    assert opt.get_step() == 5 and opt.plan.schedule_overrun() == 0
     for step, lr in ((6, lrs[5]), (7, lrs[5])):
         opt.plan.grad_norm(0.5)
-        opt.step_scheduled(fused_clip=True)
-        torch.cuda.synchronize()
         if step == 6:
+            opt.step_scheduled(fused_clip=True)
+            torch.cuda.synchronize()
             check(6, lr)
-            assert opt.plan.schedule_position() == (6, 6)
+            assert opt.plan.schedule_position() == (6, 6) and opt.get_step() == 6
+            assert opt.plan.schedule_overrun() == 0
+            with pytest.raises(RuntimeError):
+                opt.step_scheduled(fused_clip=True)              # the table is used up: the mirror refuses
+            assert opt.get_step() == 6
         else:
+            opt.plan.adamw_scheduled(B.CLIP_FUSED)
+            torch.cuda.synchronize()
             # exhausted: the last entry (step 6's bias corrections and rate) is used again
             norm, scale, _ = opt.plan.norm_read()
             bc1, bc2 = O.bias_correction(0.9, 6), O.bias_correction(0.999, 6)
@@ -513,9 +522,65 @@ def test_scheduled_steps_replay_without_the_host(O, L, host, B, torch_gpu):
                 fn(*args, h["p"], h["g"], h["m"], h["v"], lr, 0.9, 0.999, 1e-8, wd, bc1, bc2, clip_scale=scale)
             assert compare(st, hs, "step beyond the table") == 0
             assert opt.plan.schedule_position() == (6, 6)
+            assert opt.plan.schedule_overrun() == 1
     # a new upload starts again at its first entry
     opt.upload_schedule([2e-4])
-    assert opt.plan.schedule_position() == (0, 1)
+    assert opt.plan.schedule_position() == (0, 1) and opt.plan.schedule_overrun() == 0
+
+
+def test_one_recorded_step_replays_through_three_uploaded_windows(O, L, host, B, torch_gpu):
+    """The reference sets a new learning rate from its scheduler before every step of the whole run
+    (include/training/trainer.h:193-194, optimizer.h:120-122).  Here: norm + fused-clip scheduled update recorded
+    ONCE as a HIP graph after the first upload, then replayed through window 1 (3 steps), a LONGER window 2
+    (7 steps, the table is reallocated) and a shorter window 3 (2 steps), with nothing but the uploads and new
+    gradients coming from the host.  Every one of the 12 steps equals the oracle's step with the scheduler's rate
+    and the bias corrections of its step number; the position is right after every step and never passes the
+    table's length; no step overruns its table."""
+    torch = torch_gpu
+    specs = L.qwen3_tensor_list(MINI, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
+    st = host.ParamStore(specs)
+    st.fill("p", 1, 0.0, 0.02)
+    st.fill("g", 2, 0.0, 5e-3)
+    opt = host.AdamWOptimizer(st, lr=1e-3, chunk_elems=2048)
+    sched = host.LRScheduler()
+    sched.init_cosine(1e-3, 1e-5, 2, 12)
+    torch.cuda.synchronize()
+    hs = host_copy(st)
+    windows = [3, 7, 2]
+    side = torch.cuda.Stream()
+    graph = None
+    step = 0
+    for w, n in enumerate(windows):
+        lrs = [sched.get_lr(step + k) for k in range(n)]        # the rate of global step step+k, as trainer.h:193
+        assert opt.get_step() == step
+        opt.upload_schedule(lrs)
+        assert opt.plan.schedule_position() == (0, n)
+        if graph is None:
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.stream(side):
+                with torch.cuda.graph(graph, stream=side):
+                    s = torch.cuda.current_stream().cuda_stream
+                    opt.plan.grad_norm(0.5, s)
+                    opt.step_scheduled(fused_clip=True, stream=s)
+            torch.cuda.synchronize()
+            assert opt.get_step() == 0 and opt.plan.schedule_position() == (0, n)      # recording ran nothing
+        for k in range(n):
+            step += 1
+            st.fill("g", 100 + step, 0.0, 2e-3 * step)
+            torch.cuda.synchronize()
+            for i, h in enumerate(hs):
+                h["g"] = bits(st.grad(i))
+            graph.replay()
+            torch.cuda.synchronize()
+            norm, scale, sum_sq = opt.plan.norm_read()
+            assert sum_sq == O.sumsq_mirror([h["g"] for h in hs], 2048)[0] and norm > 0.5
+            oracle_step(O, L, specs, hs, step, dict(HYPER, lr=lrs[k]), clip_scale=scale)
+            assert compare(st, hs, "window %d step %d" % (w, step)) == 0
+            taken, total = opt.plan.schedule_position()
+            assert (taken, total) == (k + 1, n) and taken <= total                     # bounds of the table
+            assert opt.plan.schedule_overrun() == 0
+        opt.note_replayed_steps(n)
+    assert opt.get_step() == 12 and abs(opt.lr - sched.get_lr(11)) == 0.0
 
 
 def test_packed_norm_pass_gives_the_same_partials(O, L, host, B, torch_gpu):
@@ -547,6 +612,120 @@ def test_packed_norm_pass_gives_the_same_partials(O, L, host, B, torch_gpu):
     for pack in got:
         assert got[pack][0] == want, pack
         assert np.array_equal(got[pack][1], parts), pack
+
+
+@pytest.mark.parametrize("chunk,sizes", [
+    (512, [128, 1024, 513, 7, 65536, 129, 300_000]),             # 512-element chunks: group partials, 19 workgroups
+    (512, [512 * 32 * 64]),                                      # exactly 64 workgroups: one full ticket group
+    (512, [512 * 32 * 65 + 1]),                                  # 66 workgroups: a second, short ticket group
+    (1024, [1024 * 63, 5, 1024 * 2 + 1]),                        # 128-lane workgroups, 67 of them
+    (2048, [2048 * 200 + 3, 100]),                               # 256-lane workgroups
+    (8192, [8192 * 4100 + 77, 9000]),                            # 4,103 workgroups: beyond the automatic limit
+    (8192, [1]),                                                 # a single workgroup is its own last one
+])
+def test_norm_summed_by_the_last_workgroup_equals_the_second_launch(O, B, torch_gpu, chunk, sizes):
+    """The fixed-order sum of the partials as the tail of the first launch (the workgroup that draws the last
+    ticket adds them) against the same sum as a second launch: identical 16 result bytes, identical partials,
+    both equal to the restated order; three calls back to back each way (the tickets must be back at zero after
+    every call), also with the chunks spread over fewer workgroups, through a plan and through the entry point
+    that allocates nothing."""
+    torch = torch_gpu
+    stream = torch.cuda.current_stream().cuda_stream
+    grads = []
+    for i, n in enumerate(sizes):
+        if i % 3 == 2:
+            g = torch.empty(n, dtype=torch.float32, device="cuda:0")
+            B.fill_f32(g.data_ptr(), n, 50 + i, 0.0, 2e-3)
+        else:
+            g = torch.empty(n, dtype=torch.float16, device="cuda:0")
+            B.fill_f16(g.data_ptr(), n, 50 + i, 0.0, 5e-3)
+        grads.append(g)
+    torch.cuda.synchronize()
+    host_g = [bits(g) for g in grads]
+    want, parts = O.sumsq_mirror(host_g, chunk)
+    scale, norm = O.clip_scale(np.float32(want), 0.01)
+    descs = [B.TensorDesc(None, g.data_ptr(), None, None, None, g.numel(),
+                          B.DTYPE_F16 if g.dtype == torch.float16 else B.DTYPE_F32, B.TENSOR_GRAD_ONLY) for g in grads]
+    plan = B.Plan(descs, chunk)
+    assert plan.num_chunks == parts.size
+    results = {}
+    try:
+        for fused, grid in ((0, 0), (1, 0), (2, 0), (1, 3), (1, 64), (0, 3)):
+            B.set_tuning("norm_fused", fused)
+            B.set_tuning("norm_grid", grid)
+            for rep in range(3):
+                plan.grad_norm(0.01, stream)
+                res = read_device(plan.norm_ptr, 16).copy()
+                dev_parts = read_device(plan.partials_ptr, 8 * plan.num_chunks).view(np.float64).copy()
+                assert np.array_equal(dev_parts, parts), (fused, grid, rep)
+                results[(fused, grid, rep)] = res
+            if chunk == 512:
+                groups = read_device(plan.partials_ptr + 8 * plan.num_chunks, 8 * ((plan.num_chunks + 15) // 16))
+                assert np.array_equal(groups.view(np.float64), O.sumsq_mirror_groups(parts)), (fused, grid)
+    finally:
+        B.set_tuning("norm_fused", 2)
+        B.set_tuning("norm_grid", 0)
+    for key, res in results.items():
+        assert res.view(np.float64)[0] == want, key
+        assert res.view(np.float32)[2] == np.float32(norm) and res.view(np.float32)[3] == np.float32(scale), key
+    plan.destroy()
+    # the same through rlx_grad_norm_static: one FP16 buffer, then one FP32 buffer
+    h = [g for g in grads if g.dtype == torch.float16][0]
+    f = ([g for g in grads if g.dtype == torch.float32] or [None])[0]
+    out = torch.zeros((6, 2), dtype=torch.float64, device="cuda:0")
+    try:
+        for k, fused in enumerate((0, 1, 0, 1, 1, 0)):
+            B.set_tuning("norm_fused", fused)
+            assert B.grad_norm_static(h.data_ptr(), h.numel(), f.data_ptr() if f is not None else 0,
+                                      f.numel() if f is not None else 0, 0.01, out[k].data_ptr(), chunk, stream) == B.OK
+    finally:
+        B.set_tuning("norm_fused", 2)
+    torch.cuda.synchronize()
+    two = [bits(h)] + ([bits(f)] if f is not None else [])
+    want2, _ = O.sumsq_mirror(two, chunk)
+    for k in range(6):
+        assert read_device(out[k].data_ptr(), 8).view(np.float64)[0] == want2, k
+
+
+def test_norm_takes_the_wide_path_from_the_gradient_alignment_alone(O, L, host, B, torch_gpu):
+    """Gradients on a 16-byte boundary whose moments (and weights) start 4 bytes past one: the norm and the scale
+    pass, which touch only the gradients, must not be pushed onto their element-by-element paths by the other
+    streams' alignment, and the update must still take its own narrower path; everything equals the oracle."""
+    torch = torch_gpu
+    n = 50_000
+    p = torch.zeros(n + 8, dtype=torch.float16, device="cuda:0")
+    g = torch.zeros(n + 8, dtype=torch.float16, device="cuda:0")
+    m = torch.zeros(n + 8, dtype=torch.float32, device="cuda:0")
+    v = torch.zeros(n + 8, dtype=torch.float32, device="cuda:0")
+    B.fill_f16(p.data_ptr(), n + 8, 1, 0.0, 0.02)
+    B.fill_f16(g.data_ptr(), n + 8, 2, 0.0, 5e-3)
+    torch.cuda.synchronize()
+    assert g.data_ptr() % 16 == 0 and m.data_ptr() % 16 == 0
+    # gradient aligned; weights 2 bytes, moments 4 bytes past a 16-byte boundary
+    d = B.TensorDesc(p.data_ptr() + 2, g.data_ptr(), m.data_ptr() + 4, v.data_ptr() + 4, None, n, B.DTYPE_F16, 0)
+    plan = B.Plan([d], 2048)
+    p_before = bits(p)
+    hp, hg = p_before[1: n + 1].copy(), bits(g)[:n].copy()
+    hm, hv = np.zeros(n, np.float32), np.zeros(n, np.float32)
+    want, parts = O.sumsq_mirror([hg], 2048)
+    plan.grad_norm(0.25)
+    norm, scale, sum_sq = plan.norm_read()
+    assert sum_sq == want and norm > 0.25
+    assert np.array_equal(read_device(plan.partials_ptr, 8 * plan.num_chunks).view(np.float64), parts)
+    sp = B.StepParams(1e-3, 0.9, 0.999, 1e-8, 0.01, O.bias_correction(0.9, 1), O.bias_correction(0.999, 1))
+    plan.adamw(sp, B.CLIP_FUSED)
+    O.adamw_fp16(None, hp, hg, hm, hv, 1e-3, 0.9, 0.999, 1e-8, 0.01, sp.bias_correction1, sp.bias_correction2,
+                 clip_scale=scale)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(p)[1: n + 1], hp)
+    assert np.array_equal(bits(m)[1: n + 1], hm) and np.array_equal(bits(v)[1: n + 1], hv)
+    assert bits(p)[0] == p_before[0] and np.array_equal(bits(p)[n + 1:], p_before[n + 1:])  # neighbours untouched
+    assert bits(m)[0] == 0.0 and bits(m)[n + 1] == 0.0 and bits(v)[0] == 0.0 and bits(v)[n + 1] == 0.0
+    plan.scale_grads()
+    O.scale_half(hg, scale)
+    torch.cuda.synchronize()
+    assert np.array_equal(bits(g)[:n], hg)
+    plan.destroy()
 
 
 @pytest.mark.parametrize("n,src_off,dst_off", [(1 << 20, 0, 0), (2048 * 5 + 777, 0, 0), (300_001, 1, 0), (300_001, 0, 1),

@@ -95,6 +95,35 @@ def test_mirror_order_sum(O):
     assert O.sumsq_mirror([ones[:5]], 2048)[0] == 5.0
 
 
+def test_mirror_order_with_group_partials(O):
+    """512-element chunks: 16 consecutive chunk partials are added, in order, into one group partial before the
+    fixed-order sum.  Same pins as for the plain order (FP64 truth, known vectors, power-of-two scaling), plus the
+    grouping itself against a plain Python loop."""
+    rng = np.random.default_rng(1)
+    sizes = [128, 1024, 513, 5000, 40000, 7, 65536, 129]
+    grads = [O.fill_f16(n, 20 + i, 0.0, 1e-3) for i, n in enumerate(sizes)] + [O.fill_f32(3000, 99, 0.0, 1e-2)]
+    truth = sum(O.sum_sq_half(g) if g.dtype == np.uint16 else O.sum_sq_float(g) for g in grads)
+    s, parts = O.sumsq_mirror(grads, 512)
+    assert parts.size == sum((g.size + 511) // 512 for g in grads)
+    assert abs(s - truth) <= 1e-6 * truth
+    groups = O.sumsq_mirror_groups(parts)
+    assert groups.size == (parts.size + 15) // 16
+    for k in range(groups.size):
+        total = 0.0
+        for x in parts[16 * k: 16 * k + 16]:
+            total += float(x)                                       # Python floats are IEEE doubles
+        assert groups[k] == total
+    assert s == O.sumsq_mirror_final(groups) == O.sumsq_mirror_total(parts, 512)
+    assert O.sumsq_mirror_total(parts, 2048) == O.sumsq_mirror_final(parts)       # no grouping for other chunk sizes
+    g4 = [O.f2h(O.h2f(g) * np.float32(4.0)) if g.dtype == np.uint16 else g * np.float32(4.0) for g in grads]
+    assert O.sumsq_mirror(g4, 512)[0] == 16.0 * s
+    ones = np.full(100_000, 0x3C00, np.uint16)
+    assert O.sumsq_mirror([ones], 512)[0] == 100_000.0
+    assert O.sumsq_mirror([ones[:5]], 512)[0] == 5.0
+    perm = [np.ascontiguousarray(g[rng.permutation(g.size)]) for g in grads]
+    assert abs(O.sumsq_mirror(perm, 512)[0] - s) <= 1e-6 * s
+
+
 def test_generator(O):
     a = O.fill_f16(100_000, 77, 0.0, 1e-3)
     assert np.array_equal(a, O.fill_f16(100_000, 77, 0.0, 1e-3))
