@@ -112,6 +112,81 @@ def cpu_baseline(O, host, sample, g_clip, hyper, step, seconds=5.0):
     return out
 
 
+class HostList:
+    """Host copies of the first `count` tensors of a ParamStore whose tensors are all FP16 (weights, gradients,
+    moments as the pools hold them, padding between tensors included), for the CPU legs at full size."""
+
+    def __init__(self, st, count):
+        import numpy as np
+        import torch
+        assert all(s.dtype == 0 for s in st.specs[:count]), "HostList: FP16 tensors only"
+        self.count = count
+        self.sizes = [s.n for s in st.specs[:count]]
+        self.off_pg, self.off = st.off_pg[:count], st.off[:count]
+        end_pg, end = self.off_pg[-1] + self.sizes[-1], self.off[-1] + self.sizes[-1]
+        half = lambda t, n: t[:n].view(torch.int16).cpu().numpy().view(np.uint16)
+        self.p, self.g = half(st.p16, end_pg), half(st.g16, end_pg)
+        self.m, self.v = st.m[:end].cpu().numpy(), st.v[:end].cpu().numpy()
+        self.params = sum(self.sizes)
+        self.end_pg = end_pg
+
+    def gradients(self, st):
+        """The store's present gradients of the same tensors (another leg's gradients)."""
+        import numpy as np
+        import torch
+        return st.g16[:self.end_pg].view(torch.int16).cpu().numpy().view(np.uint16)
+
+
+def cpu_list_legs(O, host, hl, hyper, step, threads, g_clip=None, per_tensor=False, budget=4.0):
+    """The oracle's threaded step over the whole tensor list held in `hl`, timed on the host: the update alone,
+    optionally norm + clip + update with the gradients g_clip, optionally the update as one call per tensor.
+    Each leg: one untimed pass, then repeated until `budget` seconds or 20 passes."""
+    bc1, bc2 = host.bias_correction(hyper["beta1"], step), host.bias_correction(hyper["beta2"], step)
+    args = (hyper["lr"], hyper["beta1"], hyper["beta2"], hyper["eps"], hyper["wd"], bc1, bc2)
+
+    def timed(fn):
+        fn()
+        reps, t0 = 0, time.perf_counter()
+        while True:
+            fn()
+            reps += 1
+            el = time.perf_counter() - t0
+            if el >= budget or reps >= 20:
+                return el / reps * 1e3, reps
+
+    out = {"params": hl.params, "tensors": hl.count, "threads": threads}
+    ms, reps = timed(lambda: O.step_list_fp16_threaded(hl.p, hl.g, hl.m, hl.v, hl.off_pg, hl.off, hl.sizes, *args, 0.0, threads))
+    out.update(update_ms=ms, update_params_per_s=hl.params / (ms * 1e-3), update_gbps=BYTES_UPDATE * hl.params / (ms * 1e-3) / 1e9,
+               update_passes=reps)
+    if g_clip is not None:
+        ms, reps = timed(lambda: O.step_list_fp16_threaded(hl.p, g_clip, hl.m, hl.v, hl.off_pg, hl.off, hl.sizes, *args, 1.0, threads))
+        out.update(norm_clip_update_ms=ms, norm_clip_update_params_per_s=hl.params / (ms * 1e-3), norm_clip_update_passes=reps)
+    if per_tensor:
+        ms, reps = timed(lambda: O.update_per_tensor_fp16_threaded(hl.p, hl.g, hl.m, hl.v, hl.off_pg, hl.off, hl.sizes, *args, threads))
+        out.update(per_tensor_loop_update_ms=ms, per_tensor_loop_passes=reps)
+    return out
+
+
+def graph_clip_step_ms(opt, B, warmup, steps):
+    """norm + fused-clip update with device-resident hyper-parameters, recorded once as a HIP graph and replayed:
+    what a caller of rlx_plan_adamw_scheduled pays per step when nothing comes from the host.  ms per replay."""
+    import torch
+    n = 2 * (warmup + steps) + 8
+    opt.upload_schedule([opt.lr] * n)
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            s = torch.cuda.current_stream().cuda_stream
+            opt.plan.grad_norm(1.0, s)
+            opt.step_scheduled(fused_clip=True, stream=s)
+    torch.cuda.synchronize()
+    ms = time_events(graph.replay, warmup, steps)
+    opt.note_replayed_steps(warmup + steps)
+    del graph
+    return ms
+
+
 def time_events(fn, warmup, steps):
     """ms per call: `steps` calls back to back between two events on torch's current stream (the stream
     every kernel here is launched on)."""
@@ -128,8 +203,9 @@ def time_events(fn, warmup, steps):
     return a.elapsed_time(b) / steps
 
 
-def measure_workload(name, pkg, host, steps, warmup, chunk=0):
-    """Update, norm and norm + fused-clip update of one of the secondary configurations, from seeded state."""
+def measure_workload(name, pkg, host, steps, warmup, chunk=0, O=None):
+    """Update, norm and norm + fused-clip update of one of the secondary configurations, from seeded state.
+    With the oracle `O` given, also the CPU legs of this configuration at its own size (under "cpu")."""
     import torch
     B, L = pkg.binding, pkg.layout
     master = False
@@ -171,6 +247,27 @@ def measure_workload(name, pkg, host, steps, warmup, chunk=0):
 
     both = time_events(clip_step, warmup, steps)
     norm, scale, _ = opt.plan.norm_read(stream)
+    graph_ms = graph_clip_step_ms(opt, B, warmup, steps) if name != "qwen3-8b" else None
+    cpu = None
+    if O is not None and not master:
+        hyper = dict(lr=1e-5, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01)
+        t16 = min(16, host_cpus()["affinity"])
+        if name == "qwen3-8b":
+            # a slice of at least 1e9 parameters: the leading tensors (embedding, lm_head ... in list order)
+            count, tot = 0, 0
+            while tot < 1_000_000_000:
+                tot += specs[count].n
+                count += 1
+            hl = HostList(st, count)
+            cpu = cpu_list_legs(O, host, hl, hyper, 1000, t16, g_clip=hl.g, budget=4.0)
+            cpu["sample"] = "the first %d tensors of the list (%d parameters); full-size figures extrapolated by parameter count" % (count, tot)
+            for key in ("update_ms", "norm_clip_update_ms"):
+                cpu["extrapolated_full_" + key] = cpu[key] * N / tot
+        else:
+            hl = HostList(st, len(specs))
+            cpu = cpu_list_legs(O, host, hl, hyper, 1000, t16, g_clip=hl.g, per_tensor=(name == "ragged"), budget=2.0)
+            cpu["sample"] = "the whole configuration"
+        del hl
     scale_ms = time_events(lambda: opt.plan.scale_grads(stream), 1, 5)   # shrinks the gradients: last leg
     out = {
         "workload": what, "params": N, "tensors": len(specs), "bytes_per_param": bpp,
@@ -179,7 +276,10 @@ def measure_workload(name, pkg, host, steps, warmup, chunk=0):
         "norm_ms": nrm, "norm_gbps": BYTES_NORM * N / (nrm * 1e-3) / 1e9,
         "clip_step_ms": both, "clip_step_gbps": (bpp + BYTES_NORM) * N / (both * 1e-3) / 1e9,
         "grad_norm": norm, "clip_scale": scale, "scale_pass_ms": scale_ms, "unfused_clip_step_ms": both + scale_ms,
+        "graph_clip_step_ms": graph_ms,
     }
+    if cpu is not None:
+        out["cpu"] = cpu
     out["update_frac_of_peak"] = out["update_gbps"] / HBM_PEAK_GBPS
     out["clip_step_frac_of_peak"] = out["clip_step_gbps"] / HBM_PEAK_GBPS
     if name == "ragged":      # against one flat tensor of the same element count
@@ -200,6 +300,16 @@ def measure_workload(name, pkg, host, steps, warmup, chunk=0):
         out["update_vs_flat"] = upd / out["flat_update_ms"]
         out["norm_vs_flat"] = nrm / out["flat_norm_ms"]
         out["clip_step_vs_flat"] = both / out["flat_clip_step_ms"]
+        out["flat_graph_clip_step_ms"] = graph_clip_step_ms(fopt, B, warmup, steps)
+        out["graph_clip_step_vs_flat"] = graph_ms / out["flat_graph_clip_step_ms"]
+        if O is not None:      # the same element count as one flat tensor on the host
+            hl = HostList(flat, 1)
+            fcpu = cpu_list_legs(O, host, hl, dict(lr=1e-5, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01), 1000,
+                                 min(16, host_cpus()["affinity"]), budget=2.0)
+            out["cpu"]["flat_update_ms"] = fcpu["update_ms"]
+            out["cpu"]["update_vs_flat"] = out["cpu"]["update_ms"] / fcpu["update_ms"]
+            out["cpu"]["per_tensor_loop_vs_flat"] = out["cpu"]["per_tensor_loop_update_ms"] / fcpu["update_ms"]
+            del hl
         del fopt, flat
     return out
 
@@ -218,8 +328,8 @@ def workload_line(name, w, steps, warmup, B):
                      "frac": w["update_gbps"] / HBM_PEAK_GBPS, "traffic": None, "traffic_source": None,
                      "kernel": B.update_variant_name(variant), "kernel_ms": w["update_ms"],
                      "algorithmic_bytes_per_launch": w["bytes_per_param"] * w["params"]},
-        "cpu_baseline": None,
-        "measured": {k: v for k, v in w.items() if k not in ("workload", "params", "tensors")},
+        "cpu_baseline": w.get("cpu"),
+        "measured": {k: v for k, v in w.items() if k not in ("workload", "params", "tensors", "cpu")},
     }
 
 
@@ -259,7 +369,7 @@ def main():
     if args.variant is not None:
         B.set_tuning("update_variant", args.variant)
     if args.workload != "qwen3-0.6b":
-        w = measure_workload(args.workload, pkg, host, args.steps, args.warmup, args.chunk)
+        w = measure_workload(args.workload, pkg, host, args.steps, args.warmup, args.chunk, None if args.no_cpu else O)
         print(json.dumps(workload_line(args.workload, w, args.steps, args.warmup, B)), flush=True)
         return
 
@@ -345,11 +455,14 @@ def main():
     # ---- CPU baseline sample: state of the headline configuration (before the clip leg moves it on) ----
     n_s = 32 * 1024 * 1024
     sample = None if args.no_cpu else tuple(grab(k, emb, 0, n_s) for k in ("p", "g", "m", "v"))
+    # the whole configuration on the host, for the full-size CPU legs (7.2 GB)
+    host_list = None if args.no_cpu else HostList(st, len(specs))
 
     # ---- timed: norm + clip scale + fused update (configs[2]); larger gradients so that clipping is active ----
     st.fill("g", SEED_G + 1000, 0.0, 5e-3)
     stream = torch.cuda.current_stream().cuda_stream
     g_clip = None if args.no_cpu else grab("g", emb, 0, n_s)
+    g_clip_full = None if args.no_cpu else host_list.gradients(st)
 
     def clip_step():
         opt.plan.grad_norm(1.0, stream)
@@ -364,6 +477,15 @@ def main():
             "norm_ms": norm_ms, "norm_gbps": BYTES_NORM * N / (norm_ms * 1e-3) / 1e9,
             "workload": "same list, g~N(0,5e-3), max_norm=1.0: norm pass + final pass + fused-clip update"}
     clip["frac_of_peak"] = clip["achieved_gbps"] / HBM_PEAK_GBPS
+    # Where the clip step's time goes.  The plain and the fused-clip update are two kernels (the clip is a
+    # compile-time choice): the plain one on this leg's dense gradients (the headline's have 23 % exact zeros from
+    # the sparse embedding rows), and the fused-clip one alone, the scale already on the device.
+    clip["dense_update_ms"] = time_events(lambda: opt.step(), 3, max(5, args.steps // 2))
+    clip["fused_update_ms"] = time_events(lambda: opt.step(fused_clip=True), 3, max(5, args.steps // 2))
+    clip["fused_update_gbps"] = BYTES_UPDATE * N / (clip["fused_update_ms"] * 1e-3) / 1e9
+    clip["dense_update_gbps"] = BYTES_UPDATE * N / (clip["dense_update_ms"] * 1e-3) / 1e9
+    clip["ms_minus_parts"] = cev_ms - clip["norm_ms"] - clip["fused_update_ms"]
+    clip["graph_ms_per_step"] = graph_clip_step_ms(opt, B, 3, max(5, args.steps // 2))
 
     calibrate = None
     if args.calibrate:
@@ -394,7 +516,8 @@ def main():
     for name in wanted:
         t0 = time.perf_counter()
         big = name == "qwen3-8b"
-        configs[name] = measure_workload(name, pkg, host, 10 if big else min(args.steps, 50), 3 if big else min(args.warmup, 10))
+        configs[name] = measure_workload(name, pkg, host, 10 if big else min(args.steps, 50), 3 if big else min(args.warmup, 10),
+                                         O=None if args.no_cpu else O)
         torch.cuda.empty_cache()
         log("config %s: update %.4f ms, norm %.4f ms, clip step %.4f ms (%.1f s)" % (
             name, configs[name]["update_ms"], configs[name]["norm_ms"], configs[name]["clip_step_ms"],
@@ -404,6 +527,13 @@ def main():
     cpu = None
     if not args.no_cpu:
         cpu = cpu_baseline(O, host, sample, g_clip, hyper, 100)
+        # the configurations at their own sizes (the slice above stays for comparison with earlier runs)
+        cpu["configs"] = {"qwen3-0.6b": cpu_list_legs(O, host, host_list, hyper, 100, cpu["threads"], g_clip=g_clip_full)}
+        cpu["configs"]["qwen3-0.6b"]["sample"] = "the whole configuration: all 310 tensors, 7.2 GB of host state"
+        for name, w in configs.items():
+            if "cpu" in w:
+                cpu["configs"][name] = w.pop("cpu")
+        del host_list, g_clip_full
 
     # HBM bytes per launch of the update kernel as counted by the profiler: recorded beforehand with rocprofv3
     # (the counters cannot be read from inside this process), only valid for the shipped kernel and chunking
@@ -445,10 +575,12 @@ def main():
     flat = out["roofline"]
     flat["clip_step.ms"], flat["clip_step.gbps"] = clip["ms_per_step"], clip["achieved_gbps"]
     flat["clip_step.frac"], flat["clip_step.norm_ms"] = clip["frac_of_peak"], clip["norm_ms"]
+    flat["clip_step.dense_update_ms"], flat["clip_step.fused_update_ms"] = clip["dense_update_ms"], clip["fused_update_ms"]
+    flat["clip_step.graph_ms"] = clip["graph_ms_per_step"]
     for name, w in configs.items():
         for key in ("update_ms", "update_gbps", "norm_ms", "clip_step_ms", "clip_step_gbps", "flat_update_ms",
-                    "flat_norm_ms", "flat_clip_step_ms"):
-            if key in w:
+                    "flat_norm_ms", "flat_clip_step_ms", "graph_clip_step_ms", "flat_graph_clip_step_ms"):
+            if w.get(key) is not None:
                 flat["%s.%s" % (name, key)] = w[key]
     if calibrate:
         out["calibrate"] = calibrate

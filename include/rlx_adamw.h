@@ -150,7 +150,7 @@ int64_t rlx_plan_chunk_elems(const rlx_plan* plan);
  * one FP64 partial per chunk in table order (for plans with 512-element chunks, 16 consecutive
  * partials are then added, in order, into one group partial), then one workgroup adds these
  * in a fixed order, so that the result is the same bits on every run.  That last sum is a
- * second launch, or, for launches of up to 4,096 workgroups, the tail of the first one: the
+ * second launch, or, for launches of up to 256 workgroups, the tail of the first one: the
  * workgroup that finishes last (found by counting tickets, which decides who adds but not in
  * which order) does it.  Both forms give the same bits ("norm_fused" below chooses).  Writes
  * {sum_sq, norm = sqrtf((float)sum_sq), scale} to the plan's device result, where
@@ -277,7 +277,8 @@ int rlx_plan_schedule_overrun(rlx_plan* plan, int64_t* overrun, void* stream);
  *                     0 = chosen from the number of partials (default)
  *   "norm_fused"      who adds the norm's partials: 0 = always a second launch of one workgroup; 1 = the
  *                     workgroup of the first launch that finishes last, whenever that launch has at most
- *                     8,192 workgroups; 2 = that for launches of up to 4,096 workgroups (default).  Same bits.
+ *                     8,192 workgroups; 2 = that for launches of up to 256 workgroups (default; beyond one
+ *                     wave of workgroups the tickets cost more than the second launch).  Same bits.
  *   "convert_variant" rlx_fp16_to_fp32: 0 = 128 lanes x 4 elements per workgroup (default),
  *                     1 = 128 lanes x 2 elements, 2 = one element per lane, grid-stride,
  *                     3 = 256 lanes x 4 elements x 2 rounds

@@ -520,3 +520,120 @@ float orc_step_fp16_threaded(
     free(jobs);
     return norm;
 }
+
+/* ------------------------------------------------------------------ */
+/* Threaded FP16 step over a LIST of tensors for the CPU baseline: the  */
+/* concatenated index space of all tensors is split into `threads`      */
+/* contiguous ranges, so small tensors cost no thread start of their    */
+/* own.  Same arithmetic per element as orc_adamw_fp16_clip.            */
+/* ------------------------------------------------------------------ */
+
+typedef struct {
+    int64_t n_tensors;
+    uint16_t* const* model; const uint16_t* const* grad; float* const* m; float* const* v;
+    const int64_t* start;            /* start[i] = elements before tensor i; start[n_tensors] = total */
+    int64_t lo, hi;                  /* this thread's range of the concatenated index space */
+    float lr, beta1, beta2, eps, wd, bc1_inv, bc2_inv, clip_scale; int apply_clip;
+    double sumsq;
+} list_job;
+
+static int64_t list_first_tensor(const list_job* j)
+{
+    int64_t a = 0, b = j->n_tensors;             /* last i with start[i] <= lo */
+    while (b - a > 1) { int64_t mid = (a + b) / 2; if (j->start[mid] <= j->lo) a = mid; else b = mid; }
+    return a;
+}
+
+static void* list_update(void* arg)
+{
+    list_job* j = (list_job*)arg;
+    for (int64_t i = list_first_tensor(j); i < j->n_tensors && j->start[i] < j->hi; i++) {
+        int64_t lo = j->lo > j->start[i] ? j->lo - j->start[i] : 0;
+        int64_t n = j->start[i + 1] - j->start[i];
+        int64_t hi = j->hi - j->start[i] < n ? j->hi - j->start[i] : n;
+        if (hi > lo)
+            adamw_fp16_range(NULL, j->model[i], j->grad[i], j->m[i], j->v[i], lo, hi, j->lr, j->beta1, j->beta2, j->eps,
+                             j->wd, j->bc1_inv, j->bc2_inv, j->clip_scale, j->apply_clip);
+    }
+    return NULL;
+}
+
+static void* list_sumsq(void* arg)
+{
+    list_job* j = (list_job*)arg;
+    double s = 0.0;
+    for (int64_t i = list_first_tensor(j); i < j->n_tensors && j->start[i] < j->hi; i++) {
+        int64_t lo = j->lo > j->start[i] ? j->lo - j->start[i] : 0;
+        int64_t n = j->start[i + 1] - j->start[i];
+        int64_t hi = j->hi - j->start[i] < n ? j->hi - j->start[i] : n;
+        if (hi > lo) s += orc_sum_sq_half(j->grad[i] + lo, hi - lo);
+    }
+    j->sumsq = s;
+    return NULL;
+}
+
+static void run_list_jobs(list_job* jobs, int threads, void* (*fn)(void*))
+{
+    pthread_t* tid = (pthread_t*)malloc(sizeof(pthread_t) * (size_t)threads);
+    for (int t = 1; t < threads; t++) pthread_create(&tid[t], NULL, fn, &jobs[t]);
+    fn(&jobs[0]);
+    for (int t = 1; t < threads; t++) pthread_join(tid[t], NULL);
+    free(tid);
+}
+
+/*
+ * Norm (optional, max_norm > 0: FP64 sum of per-thread FP64 sums in thread order, then the clip rule of
+ * trainer.h:341-345) + update of n_tensors FP16 tensors (no master copy) on `threads` host threads.
+ * counts[i] elements each; every tensor takes the same weight decay.  Returns the pre-clip norm (0 if off).
+ */
+float orc_step_list_fp16_threaded(
+    int64_t n_tensors, uint16_t* const* model_w, const uint16_t* const* grad, float* const* m, float* const* v,
+    const int64_t* counts, float lr, float beta1, float beta2, float eps, float weight_decay,
+    float bias_correction1, float bias_correction2, float max_norm, int threads)
+{
+    if (n_tensors <= 0) return 0.0f;
+    if (threads < 1) threads = 1;
+    int64_t* start = (int64_t*)malloc(sizeof(int64_t) * (size_t)(n_tensors + 1));
+    start[0] = 0;
+    for (int64_t i = 0; i < n_tensors; i++) start[i + 1] = start[i] + (counts[i] > 0 ? counts[i] : 0);
+    const int64_t total = start[n_tensors];
+    list_job* jobs = (list_job*)calloc((size_t)threads, sizeof(list_job));
+    const int64_t per = (total + threads - 1) / threads;
+    for (int t = 0; t < threads; t++) {
+        list_job* j = &jobs[t];
+        j->n_tensors = n_tensors; j->model = model_w; j->grad = grad; j->m = m; j->v = v; j->start = start;
+        j->lo = per * t < total ? per * t : total;
+        j->hi = per * (t + 1) < total ? per * (t + 1) : total;
+        j->lr = lr; j->beta1 = beta1; j->beta2 = beta2; j->eps = eps; j->wd = weight_decay;
+        j->bc1_inv = 1.0f / bias_correction1; j->bc2_inv = 1.0f / bias_correction2;
+        j->clip_scale = 1.0f; j->apply_clip = 0;
+    }
+    float norm = 0.0f;
+    if (max_norm > 0.0f) {
+        run_list_jobs(jobs, threads, list_sumsq);
+        double s = 0.0;
+        for (int t = 0; t < threads; t++) s += jobs[t].sumsq;
+        float scale = orc_clip_scale((float)s, max_norm, &norm);
+        if (norm > max_norm)
+            for (int t = 0; t < threads; t++) { jobs[t].clip_scale = scale; jobs[t].apply_clip = 1; }
+    }
+    run_list_jobs(jobs, threads, list_update);
+    free(jobs);
+    free(start);
+    return norm;
+}
+
+/*
+ * The update of the same list as a loop over the tensors, each tensor split over the threads by itself
+ * (orc_step_fp16_threaded without clipping): what one call per tensor costs on the host, for comparison
+ * with the single split above.  Same results.
+ */
+void orc_update_per_tensor_fp16_threaded(
+    int64_t n_tensors, uint16_t* const* model_w, const uint16_t* const* grad, float* const* m, float* const* v,
+    const int64_t* counts, float lr, float beta1, float beta2, float eps, float weight_decay,
+    float bias_correction1, float bias_correction2, int threads)
+{
+    for (int64_t i = 0; i < n_tensors; i++)
+        orc_step_fp16_threaded(NULL, model_w[i], grad[i], m[i], v[i], counts[i], lr, beta1, beta2, eps, weight_decay,
+                               bias_correction1, bias_correction2, 0.0f, threads);
+}

@@ -58,6 +58,8 @@ def _load():
         "orc_fill_f16": ([vp, i64, u64, i64, f, f, u32, i64, u32], None),
         "orc_fill_f32": ([vp, i64, u64, i64, f, f, u32, i64, u32], None),
         "orc_step_fp16_threaded": ([vp, vp, vp, vp, vp, i64] + hyper + [f, i32], f),
+        "orc_step_list_fp16_threaded": ([i64, vp, vp, vp, vp, vp] + hyper + [f, i32], f),
+        "orc_update_per_tensor_fp16_threaded": ([i64, vp, vp, vp, vp, vp] + hyper + [i32], None),
     }
     for name, (args, res) in sig.items():
         fn = getattr(lib, name)
@@ -212,3 +214,31 @@ def step_fp16_threaded(master, model, grad, m, v, lr, beta1, beta2, eps, wd, bc1
     return float(lib.orc_step_fp16_threaded(_p(master, F32), _p(model, U16), _p(grad, U16), _p(m, F32),
                                             _p(v, F32), model.size, lr, beta1, beta2, eps, wd, bc1, bc2,
                                             max_norm, threads))
+
+
+def _list_pointers(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts):
+    k = len(counts)
+    ptr = C.c_void_p * k
+    cnt = (C.c_int64 * k)(*[int(c) for c in counts])
+    model = ptr(*[_p(p_pool, U16) + 2 * int(o) for o in off_pg])
+    grad = ptr(*[_p(g_pool, U16) + 2 * int(o) for o in off_pg])
+    m = ptr(*[_p(m_pool, F32) + 4 * int(o) for o in off_state])
+    v = ptr(*[_p(v_pool, F32) + 4 * int(o) for o in off_state])
+    return k, model, grad, m, v, cnt
+
+
+def step_list_fp16_threaded(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts, lr, beta1, beta2, eps, wd,
+                            bc1, bc2, max_norm, threads):
+    """Norm (if max_norm > 0) + clip + update of a LIST of FP16 tensors that live inside four pools (FP16 weights
+    and gradients share the offsets off_pg, FP32 moments the offsets off_state; counts[i] elements each), with
+    the concatenated index space split over `threads` host threads.  In place.  Returns the pre-clip norm."""
+    k, model, grad, m, v, cnt = _list_pointers(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts)
+    return float(lib.orc_step_list_fp16_threaded(k, model, grad, m, v, cnt, lr, beta1, beta2, eps, wd, bc1, bc2,
+                                                 max_norm, threads))
+
+
+def update_per_tensor_fp16_threaded(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts, lr, beta1, beta2, eps,
+                                    wd, bc1, bc2, threads):
+    """The same update as a loop over the tensors, each split over the threads by itself."""
+    k, model, grad, m, v, cnt = _list_pointers(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts)
+    lib.orc_update_per_tensor_fp16_threaded(k, model, grad, m, v, cnt, lr, beta1, beta2, eps, wd, bc1, bc2, threads)

@@ -654,23 +654,35 @@ __device__ __forceinline__ double fixed_order_sum(const double* vals, int64_t n,
     return lds[0];
 }
 
+// A value that the workgroup finishing last will add up: stored past the caches that other workgroups' loads
+// could miss it in (a device-scope store).
+__device__ __forceinline__ void publish(double* slot, double x) {
+    __hip_atomic_store(slot, x, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 // True in every lane of exactly one workgroup of the launch: the one that takes its ticket last.  Everything the
-// final sum reads must have been stored by lanes of the workgroup's first wavefront before the call.  Two levels
-// of counters (64 workgroups share a first-level counter, the last of each 64 takes a second-level ticket), so
-// that thousands of workgroups finishing together do not queue on one address.  Whoever draws a counter's last
-// ticket puts the counter back to zero for the next launch.
+// final sum reads must have been stored with publish() by lanes of the workgroup's first wavefront before the call.
+// Two levels of counters (64 workgroups share a first-level counter, the last of each 64 takes a second-level
+// ticket), so that thousands of workgroups finishing together do not queue on one address (one counter for
+// all: 12 ns per workgroup, 100 us for 8,192).  Whoever draws a counter's last ticket puts the counter back to
+// zero for the next launch.
+// Ordering: the published values are device-scope stores, the wavefront waits until they have been acknowledged
+// and only then takes its ticket; the last workgroup reads them with device-scope loads after its ticket has
+// come back.  A full device-scope fence in front of the ticket would do as well, but it writes the whole L2 back
+// and measured 67 ns per workgroup, one after the other across the device (550 us for 8,192 workgroups).
 __device__ __forceinline__ bool last_workgroup(uint32_t* tickets, int* lds_flag) {
     if (threadIdx.x < 64) {
-        __threadfence();                    // this wavefront's partials are visible device-wide before its ticket
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        wait_for_memory();                  // this wavefront's published values have arrived before its ticket is taken
         if (threadIdx.x == 0) {
             const uint32_t n_wg = gridDim.x, grp = blockIdx.x / kTicketGroup;
             const uint32_t n_grp = (n_wg + kTicketGroup - 1) / kTicketGroup;
             const uint32_t in_grp = grp + 1 < n_grp ? (uint32_t)kTicketGroup : n_wg - grp * kTicketGroup;
             uint32_t* c1 = tickets + (size_t)(1 + grp) * kTicketStride;
             int last = 0;
-            if (__hip_atomic_fetch_add(c1, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == in_grp - 1) {
+            if (__hip_atomic_fetch_add(c1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == in_grp - 1) {
                 __hip_atomic_store(c1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (__hip_atomic_fetch_add(tickets, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT) == n_grp - 1) {
+                if (__hip_atomic_fetch_add(tickets, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_grp - 1) {
                     __hip_atomic_store(tickets, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
                     last = 1;
                 }
@@ -680,7 +692,7 @@ __device__ __forceinline__ bool last_workgroup(uint32_t* tickets, int* lds_flag)
     }
     __syncthreads();
     const bool last = *lds_flag != 0;
-    if (last) __threadfence();              // what the other workgroups released is visible to this one's loads
+    if (last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     return last;
 }
 
@@ -828,7 +840,8 @@ __global__ __launch_bounds__(BLOCK * PACK) void sumsq_partials_kernel(
                 double total = 0.0;
 #pragma unroll
                 for (int w = 0; w < BLOCK / 64; w++) total += (double)wave_sum[w];
-                partials[c] = total;
+                if constexpr (FUSED) publish(&partials[c], total);
+                else partials[c] = total;
             }
             __syncthreads();
         }
@@ -941,7 +954,8 @@ __global__ __launch_bounds__(64 * WAVES) void sumsq_small_chunks_kernel(
             double total = 0.0;
 #pragma unroll
             for (int k = 0; k < kGroupChunks; k++) total += chunk_sum[threadIdx.x * kGroupChunks + k];
-            groups[grp] = total;
+            if constexpr (FUSED) publish(&groups[grp], total);
+            else groups[grp] = total;
         }
     }
     if constexpr (FUSED) {
@@ -1189,7 +1203,7 @@ struct Tuning {
     std::atomic<int64_t> final_batch{0};    // loads in flight per lane in the second pass of the norm; 0 = by the number of partials
     std::atomic<int64_t> norm_fused{2};     // the fixed-order sum of the partials: 0 = always a second launch, 1 = by the
                                             // workgroup of the first launch that finishes last whenever that launch
-                                            // has at most 8,192 workgroups, 2 = that up to 4,096 workgroups (default)
+                                            // has at most 8,192 workgroups, 2 = that up to 256 workgroups (default)
 } g_tuning;
 
 constexpr int kNumUpdateVariants = 17;
@@ -1561,8 +1575,13 @@ struct NormWork {
 
 inline int64_t norm_groups(int64_t n_chunks) { return (n_chunks + kGroupChunks - 1) / kGroupChunks; }
 
-// Workgroups up to which the automatic choice ("norm_fused" = 2) lets the last workgroup add the partials.
-constexpr int64_t kAutoFusedWgs = 4096;
+// Workgroups up to which the automatic choice ("norm_fused" = 2) lets the last workgroup add the partials: as
+// many as the device has CUs.  Measured on flat FP16 tensors of 8,192-element chunks, norm + fused-clip update:
+// 64 and 128 workgroups 12.5 us against 16.0 us with the sum as a second launch (the norm alone 5.8 against
+// 6.3); 256: 15.6 either way; 512: 22.1 against 21.3; 1,536: 52.4 against 51.4 (the norm alone 8.8 against 6.6);
+// the 1,202 workgroups of the 4,096-tensor list: 14.2 against 11.9 for the norm alone.  Beyond one wave of
+// workgroups the tickets cost more than the second launch.
+constexpr int64_t kAutoFusedWgs = 256;
 
 template <bool NT, bool POOLS, int BLOCK>
 hipError_t launch_partials(const NormWork& w, int64_t grid, bool fused, const NormTail& tail, hipStream_t s) {

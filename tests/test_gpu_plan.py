@@ -654,14 +654,22 @@ def test_norm_summed_by_the_last_workgroup_equals_the_second_launch(O, B, torch_
             B.set_tuning("norm_fused", fused)
             B.set_tuning("norm_grid", grid)
             for rep in range(3):
+                # every call sees new values (all gradients doubled, which multiplies every partial and the sum
+                # by exactly 4): a sum that picked up a partial of the call before would show
                 plan.grad_norm(0.01, stream)
                 res = read_device(plan.norm_ptr, 16).copy()
                 dev_parts = read_device(plan.partials_ptr, 8 * plan.num_chunks).view(np.float64).copy()
-                assert np.array_equal(dev_parts, parts), (fused, grid, rep)
-                results[(fused, grid, rep)] = res
-            if chunk == 512:
-                groups = read_device(plan.partials_ptr + 8 * plan.num_chunks, 8 * ((plan.num_chunks + 15) // 16))
-                assert np.array_equal(groups.view(np.float64), O.sumsq_mirror_groups(parts)), (fused, grid)
+                assert np.array_equal(dev_parts, parts * 4.0 ** rep), (fused, grid, rep)
+                assert res.view(np.float64)[0] == want * 4.0 ** rep, (fused, grid, rep)
+                if rep == 0:
+                    results[(fused, grid)] = res
+                    if chunk == 512:
+                        groups = read_device(plan.partials_ptr + 8 * plan.num_chunks, 8 * ((plan.num_chunks + 15) // 16))
+                        assert np.array_equal(groups.view(np.float64), O.sumsq_mirror_groups(parts)), (fused, grid)
+                for g in grads:
+                    g.mul_(2.0)
+            for g in grads:
+                g.mul_(0.125)
     finally:
         B.set_tuning("norm_fused", 2)
         B.set_tuning("norm_grid", 0)

@@ -266,3 +266,34 @@ def test_tolerances_cover_a_reference_binary_built_with_fma_contraction(O):
         same_sign = (p & 0x8000) == (p_fma & 0x8000)
         assert ulp[same_sign].max() <= 1 and (ulp[~same_sign] <= 1).all(), step      # +-0 against each other at most
     assert worst_m <= 1e-6 and worst_v <= 1e-6, (worst_m, worst_v)
+
+
+def test_threaded_list_step_equals_per_tensor_steps(O):
+    """The CPU baseline's step over a tensor list (one split of the concatenated index space over the threads)
+    gives, for any thread count, the bits of the plain per-tensor update; with clipping, the norm is within the
+    path's 1e-5 of the FP64 sum and the scaled, re-rounded gradients are the ones the update sees."""
+    sizes = [128, 1024, 5000, 7, 65536, 300]
+    off, total = [], 0
+    for n in sizes:
+        off.append(total)
+        total += (n + 127) // 128 * 128
+    p, g = O.fill_f16(total, 1, 0.0, 0.02), O.fill_f16(total, 2, 0.0, 5e-3)
+    m, v = O.fill_f32(total, 3, 0.0, 1e-4), O.fill_f32(total, 4, 1e-8, 1e-8, flags=O.FILL_ABS)
+    args = (1e-3, 0.9, 0.999, 1e-8, 0.01, 0.1, 0.001)
+    for max_norm in (0.0, 0.01):
+        ref = [x.copy() for x in (p, m, v)]
+        ssq = sum(O.sum_sq_half(np.ascontiguousarray(g[o: o + n])) for o, n in zip(off, sizes))
+        scale, norm = O.clip_scale(np.float32(ssq), max_norm) if max_norm > 0 else (None, 0.0)
+        for o, n in zip(off, sizes):
+            parts = [np.ascontiguousarray(x[o: o + n]) for x in ref]
+            O.adamw_fp16(None, parts[0], np.ascontiguousarray(g[o: o + n]), parts[1], parts[2], *args,
+                         clip_scale=scale if max_norm > 0 and norm > max_norm else None)
+            for x, part in zip(ref, parts):
+                x[o: o + n] = part
+        for threads in (1, 3, 16):
+            q = [x.copy() for x in (p, g, m, v)]
+            got = O.step_list_fp16_threaded(q[0], q[1], q[2], q[3], off, off, sizes, *args, max_norm, threads)
+            assert np.array_equal(q[0], ref[0]) and np.array_equal(q[1], g), threads
+            assert np.array_equal(q[2].view(np.uint32), ref[1].view(np.uint32)), threads
+            assert np.array_equal(q[3].view(np.uint32), ref[2].view(np.uint32)), threads
+            assert abs(got - norm) <= 1e-5 * max(norm, 1e-30), threads
