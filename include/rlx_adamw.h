@@ -279,6 +279,11 @@ int rlx_plan_schedule_overrun(rlx_plan* plan, int64_t* overrun, void* stream);
  *                     workgroup of the first launch that finishes last, whenever that launch has at most
  *                     8,192 workgroups; 2 = that for launches of up to 256 workgroups (default; beyond one
  *                     wave of workgroups the tickets cost more than the second launch).  Same bits.
+ *   "norm_keep_mb"    > 0: the norm walks its chunks from the last to the first and reads the first that many
+ *                     MB of gradients (the last it reads) with ordinary instead of non-temporal loads, so that
+ *                     they are still in the last-level cache when the update starts; 0 = off (default).  Same bits.
+ *   "update_reverse"  1 = the fused-clip update walks its tiles from the end of the table to its start (to meet
+ *                     what a forward norm read last); 0 = off (default).  Same bits.
  *   "convert_variant" rlx_fp16_to_fp32: 0 = 128 lanes x 4 elements per workgroup (default),
  *                     1 = 128 lanes x 2 elements, 2 = one element per lane, grid-stride,
  *                     3 = 256 lanes x 4 elements x 2 rounds

@@ -501,7 +501,7 @@ __global__ __launch_bounds__(BLOCK) void adamw_rounds_kernel(
 // SINGLE: one flat tensor passed by value (the operator API); otherwise the plan's records.
 // ---------------------------------------------------------------------------------------
 
-template <int E, int BLOCK, int K, bool SINGLE, int SP, int PH, bool NTL, bool CLIP>
+template <int E, int BLOCK, int K, bool SINGLE, int SP, int PH, bool NTL, bool CLIP, bool REV = false>
 __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
     const ChunkRec* __restrict__ recs, ChunkRec single, int64_t single_n, int64_t first_tile, int64_t n_tiles,
     int tiles_per_chunk_log2, Hyper h, const rlx_step_params* __restrict__ dev_params,
@@ -513,8 +513,9 @@ __global__ __launch_bounds__(BLOCK) void adamw_tile_kernel(
         const int64_t grp = b / (8 * K), r = b % (8 * K);
         b = grp * (8 * K) + (r % 8) * K + (r / 8);
     }
-    const int64_t tile = first_tile + b;
+    int64_t tile = first_tile + b;
     if (tile >= n_tiles) return;
+    if constexpr (REV) tile = n_tiles - 1 - tile;     // from the end of the table to its start
 
     ChunkRec r;
     int64_t off;         // first element of the tile, relative to r's pointers
@@ -599,6 +600,10 @@ struct NormTail {
     NormResult* out;
     uint32_t* tickets;           // [0]: second-level counter; [(1 + g) * kTicketStride]: counter of workgroups
                                  // 64g .. 64g+63.  All zero between launches.
+    int64_t plain_below;         // > 0: the launch walks the chunks from the last to the first, and chunks with an
+                                 // index below this are read with ordinary instead of non-temporal loads, so that
+                                 // what the norm reads last, the start of the gradients, is what stays in the
+                                 // last-level cache for the update that follows
 };
 
 // The sum, the norm and the clip scale (trainer.h:341-345: strict '>' and +1e-6f in the denominator).
@@ -823,11 +828,14 @@ __global__ __launch_bounds__(BLOCK * PACK) void sumsq_partials_kernel(
     const int tid = PACK == 1 ? (int)threadIdx.x : (int)(threadIdx.x & 63);
     const int sub = PACK == 1 ? 0 : __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
 
-    for (int64_t c = (int64_t)blockIdx.x * PACK + sub; c < n_chunks; c += (int64_t)gridDim.x * PACK) {
+    for (int64_t i = (int64_t)blockIdx.x * PACK + sub; i < n_chunks; i += (int64_t)gridDim.x * PACK) {
+        const int64_t c = tail.plain_below > 0 ? n_chunks - 1 - i : i;      // the slot is the chunk's: same sum either way
         ChunkRec r;
         if constexpr (POOLS) r = pool_chunk(pools, c);
         else r = recs[c];
-        float acc = chunk_lane_sumsq<NT, BLOCK>(r, tid);
+        float acc;
+        if (NT && c < tail.plain_below) acc = chunk_lane_sumsq<false, BLOCK>(r, tid);
+        else acc = chunk_lane_sumsq<NT, BLOCK>(r, tid);
 #pragma unroll
         for (int mask = 32; mask >= 1; mask >>= 1) acc = acc + __shfl_xor(acc, mask, 64);
         if constexpr (BLOCK == 64) {
@@ -1201,6 +1209,9 @@ struct Tuning {
                                             // 2 = thirty-two (four per wavefront, the default), 3 = sixteen
     std::atomic<int64_t> convert_variant{0};
     std::atomic<int64_t> final_batch{0};    // loads in flight per lane in the second pass of the norm; 0 = by the number of partials
+    std::atomic<int64_t> norm_keep_mb{0};   // > 0: the norm walks its chunks backwards and reads the first that many MB of
+                                            // gradients, last in time, with ordinary loads (they stay cached for the update)
+    std::atomic<int64_t> update_reverse{0}; // 1: the fused-clip update walks the tile table from its end to its start
     std::atomic<int64_t> norm_fused{2};     // the fixed-order sum of the partials: 0 = always a second launch, 1 = by the
                                             // workgroup of the first launch that finishes last whenever that launch
                                             // has at most 8,192 workgroups, 2 = that up to 256 workgroups (default)
@@ -1306,7 +1317,13 @@ hipError_t launch_variant(const ChunkRec* recs, const ChunkRec& single, int64_t 
     for (int64_t first = 0; first < n_tiles; first += kMaxTilesPerLaunch) {
         int64_t here = n_tiles - first < kMaxTilesPerLaunch ? n_tiles - first : kMaxTilesPerLaunch;
         here = (here + 8 * K - 1) / (8 * K) * (8 * K);   // whole swizzle groups; the excess exits at once
-        if (norm)
+        bool reversed = false;
+        if constexpr (E == 2 && BLOCK == 128 && K == 1 && !SINGLE && SP == 1 && NTL) reversed = norm && g_tuning.update_reverse != 0;
+        if (reversed) {
+            if constexpr (E == 2 && BLOCK == 128 && K == 1 && !SINGLE && SP == 1 && NTL)
+                adamw_tile_kernel<E, BLOCK, K, SINGLE, SP, PH, NTL, true, true><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(
+                    recs, single, single_n, first, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
+        } else if (norm)
             adamw_tile_kernel<E, BLOCK, K, SINGLE, SP, PH, NTL, true><<<dim3((unsigned)here), dim3(BLOCK), 0, s>>>(
                 recs, single, single_n, first, n_tiles, tpc_log2, h, dev_params, norm, step_flags);
         else
@@ -1618,6 +1635,10 @@ int launch_norm_nt(const NormWork& w, float max_norm, hipStream_t s) {
     tail.max_norm = max_norm;
     tail.out = w.result;
     tail.tickets = w.tickets;
+    // "norm_keep_mb": that many MB of gradients at the start of the table (FP16 chunks assumed) are read last and
+    // with ordinary loads
+    const int64_t keep_mb = g_tuning.norm_keep_mb;
+    tail.plain_below = keep_mb > 0 && !grouped ? (keep_mb << 20) / (w.chunk_elems * 2) + 1 : 0;
     const auto want_fused = [&](int64_t grid) {
         return grid <= kMaxFusedWgs && (norm_fused == 1 || (norm_fused == 2 && grid <= kAutoFusedWgs));
     };
@@ -2121,6 +2142,11 @@ int rlx_set_tuning(const char* key, int64_t value) {
         if (value > 2) return RLX_ERR_INVALID_ARG;
         g_tuning.norm_fused = value;
     }
+    else if (!strcmp(key, "update_reverse")) g_tuning.update_reverse = value ? 1 : 0;
+    else if (!strcmp(key, "norm_keep_mb")) {
+        if (value > 4096) return RLX_ERR_INVALID_ARG;
+        g_tuning.norm_keep_mb = value;
+    }
     else if (!strcmp(key, "convert_variant")) {
         if (value >= kNumConvertVariants) return RLX_ERR_INVALID_ARG;
         g_tuning.convert_variant = value;
@@ -2137,6 +2163,8 @@ int64_t rlx_get_tuning(const char* key) {
     if (!strcmp(key, "convert_variant")) return g_tuning.convert_variant;
     if (!strcmp(key, "final_batch")) return g_tuning.final_batch;
     if (!strcmp(key, "norm_fused")) return g_tuning.norm_fused;
+    if (!strcmp(key, "update_reverse")) return g_tuning.update_reverse;
+    if (!strcmp(key, "norm_keep_mb")) return g_tuning.norm_keep_mb;
     return -1;
 }
 

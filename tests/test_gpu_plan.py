@@ -321,6 +321,39 @@ def test_every_tile_shape_and_chunk_size_gives_the_same_bits(L, host, B, torch_g
         assert all(torch.equal(a, b) for a, b in zip(results[0], r))
 
 
+def test_cache_aware_orders_give_the_same_bits(L, host, B, torch_gpu):
+    """The two orders meant to let the update find the gradients that the norm read last still in the last-level
+    cache (the norm walking its chunks backwards with ordinary loads on the stretch it reads last; the fused-clip
+    update walking its tiles backwards) change neither the norm's result nor any bit of the state: every chunk's
+    partial keeps its slot, every tile its arithmetic."""
+    torch = torch_gpu
+    specs = [L.TensorSpec("a", 300_001, L.DTYPE_F16, 0, 0), L.TensorSpec("b", 2049, L.DTYPE_F32, 0, 0),
+             L.TensorSpec("c", 131, L.DTYPE_F16, L.NO_DECAY, 0), L.TensorSpec("d", 9000, L.DTYPE_F16, 0, 0)]
+    results = {}
+    try:
+        for chunk in (8192, 1024):
+            for keep_mb, reverse in [(0, 0), (1, 0), (0, 1), (1, 1), (4096, 1)]:
+                B.set_tuning("norm_keep_mb", keep_mb)
+                B.set_tuning("update_reverse", reverse)
+                st = host.ParamStore(specs)
+                st.fill("p", 1, 0.0, 0.02)
+                st.fill("g", 2, 0.0, 5e-3)
+                opt = host.AdamWOptimizer(st, lr=1e-3, chunk_elems=chunk)
+                norm = host.training_step(opt, 0.05, fused_clip=True)
+                st.fill("g", 3, 0.0, 5e-3)
+                norm2 = host.training_step(opt, 0.05, fused_clip=True, zero_grads=True)
+                torch.cuda.synchronize()
+                results[(chunk, keep_mb, reverse)] = (np.float32(norm), np.float32(norm2),
+                                                      [t.clone() for t in (st.p16, st.p32, st.m, st.v)])
+    finally:
+        B.set_tuning("norm_keep_mb", 0)
+        B.set_tuning("update_reverse", 0)
+    for (chunk, keep_mb, reverse), (norm, norm2, state) in results.items():
+        base = results[(chunk, 0, 0)]                    # the order of the sum, and so its bits, belong to the chunk size
+        assert norm == base[0] and norm2 == base[1], (chunk, keep_mb, reverse)
+        assert all(torch.equal(a, b) for a, b in zip(base[2], state)), (chunk, keep_mb, reverse)
+
+
 def test_unaligned_tensors_in_a_plan(O, L, host, B, torch_gpu):
     """Tensors that start at odd element offsets take the element-by-element path."""
     torch = torch_gpu
