@@ -152,7 +152,9 @@ int64_t rlx_plan_chunk_elems(const rlx_plan* plan);
  * in a fixed order, so that the result is the same bits on every run.  That last sum is a
  * second launch, or, for launches of up to 256 workgroups, the tail of the first one: the
  * workgroup that finishes last (found by counting tickets, which decides who adds but not in
- * which order) does it.  Both forms give the same bits ("norm_fused" below chooses).  Writes
+ * which order) does it.  Both forms give the same bits ("norm_fused" below chooses).  The tickets live in the
+ * plan and are zero between launches: norm launches of ONE plan must not overlap (two streams, two threads),
+ * or the counters can be left non-zero and later norms of that plan never complete their sum.  Writes
  * {sum_sq, norm = sqrtf((float)sum_sq), scale} to the plan's device result, where
  * scale = max_norm / (norm + 1e-6f) iff norm > max_norm, else 1.0f (a NaN norm gives
  * 1.0f, as the reference's comparison does; max_norm = INFINITY measures without clipping).
@@ -177,8 +179,7 @@ const double* rlx_plan_partials_device_ptr(const rlx_plan* plan);
  * The same two-pass norm and clip rule over two flat gradient buffers (an FP16 one, then an FP32 one: the
  * shape of half_pool / float_pool) without a plan and without allocating anything.  It has no counterpart
  * in the reference; it is for callers that cannot allocate: code under HIP graph capture, tight serving
- * loops, harnesses that forbid hipMalloc.  The FP64 partials (and the ticket counters of the one-launch form)
- * go to a 2.2 MiB array that is part of
+ * loops, harnesses that forbid hipMalloc.  The FP64 partials go to a 2.1 MiB array that is part of
  * the library's device image (every GPU the library runs on holds it until the process ends), so at most
  * 262,144 chunks fit: more returns RLX_ERR_TOO_LARGE (chunk_elems = 0 chooses the chunk as rlx_plan_create
  * would for these two tensors, which covers about 17e9 elements; otherwise a power of two >= 512).
@@ -187,9 +188,9 @@ const double* rlx_plan_partials_device_ptr(const rlx_plan* plan);
  * Either buffer may be empty (n = 0).  Calls no hipMalloc, hipFree or other allocating routine; the first call
  * on a device looks up the array's address there (make that call outside a graph capture).  All calls on one
  * GPU share the array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream
- * do not.  The partials need not start at zero: every call writes each slot that it later reads.  The ticket
- * counters must, and do: they are zero in the image and the workgroup that draws a counter's last ticket sets
- * it back to zero, so every call that runs to its end leaves them at zero for the next.
+ * do not.  Nothing in the array has to start at zero: every call writes each slot that it later reads (this
+ * entry point always adds the partials in a second launch, whatever "norm_fused" says: the one-launch form keeps
+ * counters that must be zero between calls, which overlapping calls on a shared array could spoil for good).
  */
 int rlx_grad_norm_static(const uint16_t* half_grads, int64_t n_half, const float* float_grads, int64_t n_float,
                          int64_t chunk_elems, float max_norm, void* result_dev, void* stream);

@@ -41,15 +41,16 @@
 #include "rlx_adamw.h"
 
 // Intermediate sums of rlx_grad_norm_static, the entry point for callers that cannot allocate: part of the
-// library's device image (2.2 MiB on every GPU the library runs on, until the process ends).  Layout, in
+// library's device image (2.1 MiB on every GPU the library runs on, until the process ends).  Layout, in
 // doubles: [0, 2^18) per-chunk FP64 partials; [2^18, 2^18 + 2^14) group partials (one per 16 chunks, used with
-// 512-element chunks); then 16.5 KiB of 32-bit ticket counters, which start at zero in the image and which every
-// launch leaves at zero again.  The name stands for the array only in device code; host code uses the address
-// that hipGetSymbolAddress returns for the current device (static_scratch below), never the name.
+// 512-element chunks).  Nothing in it has to start at zero: every call writes each slot that it later reads (the
+// entry point always adds the partials in a second launch; the one-launch form needs counters that must be zero
+// between calls, and calls that overlap on this shared array could leave them otherwise for good).  The name
+// stands for the array only in device code; host code uses the address that hipGetSymbolAddress returns for the
+// current device (static_scratch below), never the name.
 constexpr int64_t kStaticMaxPartials = 1 << 18;
 constexpr int64_t kStaticMaxGroups = kStaticMaxPartials / 16;
-constexpr int64_t kStaticTicketDoubles = (8192 / 64 + 1) * 32 / 2;      // kTicketWords 32-bit words
-static __device__ __align__(256) double scratch[kStaticMaxPartials + kStaticMaxGroups + kStaticTicketDoubles];
+static __device__ __align__(256) double scratch[kStaticMaxPartials + kStaticMaxGroups];
 
 namespace {
 
@@ -589,8 +590,7 @@ constexpr int kTicketGroup = 64;              // workgroups per first-level tick
 constexpr int kTicketStride = 32;             // 32-bit words from one counter to the next (128 bytes: a line each)
 constexpr int64_t kMaxFusedWgs = 8192;        // largest grid whose last workgroup adds the partials itself
 constexpr int64_t kTicketWords = (kMaxFusedWgs / kTicketGroup + 1) * kTicketStride;
-static_assert(kStaticTicketDoubles * 2 == kTicketWords && kStaticMaxGroups * kGroupChunks == kStaticMaxPartials,
-              "the static scratch holds the partials, their groups and the tickets of the largest call");
+static_assert(kStaticMaxGroups * kGroupChunks == kStaticMaxPartials, "the static scratch holds the partials and their groups");
 
 // What the workgroup that finishes last needs for step 3.
 struct NormTail {
@@ -1586,7 +1586,7 @@ struct NormWork {
     int64_t n_chunks, chunk_elems;
     double* partials;            // one per chunk
     double* groups;              // one per 16 chunks; only used with 512-element chunks
-    uint32_t* tickets;           // kTicketWords words, all zero between launches
+    uint32_t* tickets;           // kTicketWords words, all zero between launches; null: never the one-launch form
     NormResult* result;
 };
 
@@ -1639,8 +1639,8 @@ int launch_norm_nt(const NormWork& w, float max_norm, hipStream_t s) {
     // with ordinary loads
     const int64_t keep_mb = g_tuning.norm_keep_mb;
     tail.plain_below = keep_mb > 0 && !grouped ? (keep_mb << 20) / (w.chunk_elems * 2) + 1 : 0;
-    const auto want_fused = [&](int64_t grid) {
-        return grid <= kMaxFusedWgs && (norm_fused == 1 || (norm_fused == 2 && grid <= kAutoFusedWgs));
+    const auto want_fused = [&](int64_t grid) {      // no ticket counters (w.tickets null): always a second launch
+        return w.tickets && grid <= kMaxFusedWgs && (norm_fused == 1 || (norm_fused == 2 && grid <= kAutoFusedWgs));
     };
     bool fused = false;
     hipError_t e = hipSuccess;
@@ -1992,7 +1992,7 @@ int rlx_grad_norm_static(const uint16_t* half_grads, int64_t n_half, const float
     memset(&w, 0, sizeof(w));
     w.pools = pp; w.n_chunks = n_chunks; w.chunk_elems = chunk_elems;
     w.partials = base; w.groups = base + kStaticMaxPartials;
-    w.tickets = (uint32_t*)(base + kStaticMaxPartials + kStaticMaxGroups);
+    w.tickets = nullptr;
     w.result = (NormResult*)result_dev;
     return launch_norm<true>(w, max_norm, (hipStream_t)stream);
 }

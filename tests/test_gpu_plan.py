@@ -710,7 +710,8 @@ def test_norm_summed_by_the_last_workgroup_equals_the_second_launch(O, B, torch_
         assert res.view(np.float64)[0] == want, key
         assert res.view(np.float32)[2] == np.float32(norm) and res.view(np.float32)[3] == np.float32(scale), key
     plan.destroy()
-    # the same through rlx_grad_norm_static: one FP16 buffer, then one FP32 buffer
+    # the same through rlx_grad_norm_static (always the second launch, whatever the tuning says): one FP16 buffer,
+    # then one FP32 buffer
     h = [g for g in grads if g.dtype == torch.float16][0]
     f = ([g for g in grads if g.dtype == torch.float32] or [None])[0]
     out = torch.zeros((6, 2), dtype=torch.float64, device="cuda:0")
