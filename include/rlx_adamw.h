@@ -273,7 +273,7 @@ int rlx_plan_schedule_overrun(rlx_plan* plan, int64_t* overrun, void* stream);
  *   "norm_grid"       0 = one workgroup per chunk, >0 = that many persistent workgroups
  *   "norm_nt"         1 = non-temporal loads in the norm pass (default), 0 = plain
  *   "norm_pack"       512-element chunks per workgroup in the norm pass: 0 = one, 1 = eight (one per
- *                     wavefront), 2 = thirty-two (four per wavefront, default), 3 = sixteen
+ *                     wavefront), 2 = thirty-two (four per wavefront), 3 = sixteen (two per wavefront, default)
  *   "final_batch"     loads that a lane of the norm's second pass keeps in flight: 8, 16, 32, 40, or
  *                     0 = chosen from the number of partials (default)
  *   "norm_fused"      who adds the norm's partials: 0 = always a second launch of one workgroup; 1 = the

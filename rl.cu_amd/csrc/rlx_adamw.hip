@@ -1205,8 +1205,9 @@ struct Tuning {
     std::atomic<int64_t> update_variant{0};
     std::atomic<int64_t> norm_grid{0};
     std::atomic<int64_t> norm_nt{1};
-    std::atomic<int64_t> norm_pack{2};      // 512-element chunks per workgroup: 0 = one, 1 = eight (a wavefront each),
-                                            // 2 = thirty-two (four per wavefront, the default), 3 = sixteen
+    std::atomic<int64_t> norm_pack{3};      // 512-element chunks per workgroup: 0 = one, 1 = eight (a wavefront each),
+                                            // 2 = thirty-two (four per wavefront), 3 = sixteen (two per wavefront,
+                                            // one group partial per workgroup: the default)
     std::atomic<int64_t> convert_variant{0};
     std::atomic<int64_t> final_batch{0};    // loads in flight per lane in the second pass of the norm; 0 = by the number of partials
     std::atomic<int64_t> norm_keep_mb{0};   // > 0: the norm walks its chunks backwards and reads the first that many MB of
@@ -1671,8 +1672,10 @@ int launch_norm_nt(const NormWork& w, float max_norm, hipStream_t s) {
             e = hipGetLastError();
         }
     } else {
-        // 512-element chunks, the default: eight wavefronts per workgroup, four (or two) chunks each
-        const int64_t per_wg = norm_pack == 3 ? 16 : 32;
+        // 512-element chunks, the default: eight wavefronts per workgroup, two (or four) chunks each.  Measured on
+        // the 4,096-tensor list, norm / norm + fused-clip update: two per wavefront 11.25 / 79.4 us, four 12.3 / 81.1,
+        // four wavefronts x four 11.9 / 80.4, sixteen wavefronts x one 14.1 / 82.1
+        const int64_t per_wg = norm_pack == 2 ? 32 : 16;
         const int64_t g = (w.n_chunks + per_wg - 1) / per_wg;
         if (g > kMaxNormGrid) return RLX_ERR_TOO_LARGE;
         fused = want_fused(g);

@@ -640,7 +640,7 @@ def test_packed_norm_pass_gives_the_same_partials(O, L, host, B, torch_gpu):
             _, _, sum_sq = opt.plan.norm_read()
             got[pack] = (sum_sq, read_device(opt.plan.partials_ptr, 8 * opt.plan.num_chunks).view(np.float64).copy())
     finally:
-        B.set_tuning("norm_pack", 2)
+        B.set_tuning("norm_pack", 3)
         B.set_tuning("final_batch", 0)
     for pack in got:
         assert got[pack][0] == want, pack
