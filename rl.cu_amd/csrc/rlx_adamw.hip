@@ -1407,8 +1407,9 @@ hipError_t launch_rounds(const ChunkRec* recs, int64_t n_chunks, int chunk_log2,
     return hipSuccess;
 }
 
-// The compiled forms of the update ("update_variant"), by number; 0 is what ships.  Every kernel has one more,
-// last template argument that the names leave out: false for the plain update, true for the fused-clip one.
+// The compiled forms of the update ("update_variant"), by number; 0 is what ships.  The names leave out the
+// template arguments behind these: whether the clip scale is applied (false for the plain update, true for the
+// fused-clip one) and, for adamw_tile_kernel, whether the tiles are walked backwards ("update_reverse").
 const char* const kVariantNames[kNumUpdateVariants] = {
     "adamw_tile_kernel<2,128,1,*,1,0|1>",      // 0: 2 elements x 128 lanes, sc1 nt stores; loads at once, or two
                                                //    at a time when the step writes four streams
