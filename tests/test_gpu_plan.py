@@ -729,6 +729,40 @@ def test_norm_summed_by_the_last_workgroup_equals_the_second_launch(O, B, torch_
         assert read_device(out[k].data_ptr(), 8).view(np.float64)[0] == want2, k
 
 
+def test_last_workgroup_sum_sees_every_partial_of_its_own_launch(B, torch_gpu):
+    """The one-launch norm relies on device-scope stores, a wait and relaxed tickets instead of a full fence: a
+    partial that the last workgroup read too early, or out of a cache, would be the value of the launch before.
+    300 launches on gradients that change every time (a new seed and a new scale, so every chunk's partial moves),
+    each followed at once by a fused-clip update that reads the scale, and each compared with the second-launch
+    form on the same gradients: all 16 result bytes identical every time."""
+    torch = torch_gpu
+    stream = torch.cuda.current_stream().cuda_stream
+    n = 8192 * 200 + 123                                          # 201 workgroups: four ticket groups, the last short
+    p = torch.zeros(n, dtype=torch.float16, device="cuda:0")
+    g = torch.empty(n, dtype=torch.float16, device="cuda:0")
+    m = torch.zeros(n, dtype=torch.float32, device="cuda:0")
+    v = torch.zeros(n, dtype=torch.float32, device="cuda:0")
+    plan = B.Plan([B.TensorDesc(p.data_ptr(), g.data_ptr(), m.data_ptr(), v.data_ptr(), None, n, B.DTYPE_F16, 0)], 8192)
+    sp = B.StepParams(1e-4, 0.9, 0.999, 1e-8, 0.0, 0.1, 0.001)
+    seen = set()
+    try:
+        for k in range(300):
+            B.fill_f16(g.data_ptr(), n, 1000 + k, 0.0, 1e-3 * (1 + k % 7), stream=stream)
+            B.set_tuning("norm_fused", 1)
+            plan.grad_norm(0.5, stream)
+            plan.adamw(sp, B.CLIP_FUSED, stream)                  # reads the scale the moment the norm has finished
+            one = read_device(plan.norm_ptr, 16).copy()
+            B.set_tuning("norm_fused", 0)
+            plan.grad_norm(0.5, stream)
+            two = read_device(plan.norm_ptr, 16).copy()
+            assert np.array_equal(one, two), (k, one.view(np.float64)[0], two.view(np.float64)[0])
+            seen.add(float(one.view(np.float64)[0]))
+    finally:
+        B.set_tuning("norm_fused", 2)
+    assert len(seen) == 300                                       # the sums did change from launch to launch
+    plan.destroy()
+
+
 def test_norm_takes_the_wide_path_from_the_gradient_alignment_alone(O, L, host, B, torch_gpu):
     """Gradients on a 16-byte boundary whose moments (and weights) start 4 bytes past one: the norm and the scale
     pass, which touch only the gradients, must not be pushed onto their element-by-element paths by the other
