@@ -97,6 +97,8 @@ def test_plan_argument_checks(B):
     assert lib.rlx_plan_schedule_upload(None, sp, 1, None) == B.ERR_INVALID_ARG
     assert lib.rlx_plan_adamw_scheduled(None, 0, None) == B.ERR_INVALID_ARG
     assert lib.rlx_plan_schedule_position(None, None, None, None) == B.ERR_INVALID_ARG
+    over = C.c_int64(-1)
+    assert lib.rlx_plan_schedule_overrun(None, C.byref(over), None) == B.ERR_INVALID_ARG and over.value == -1
     # the entry point that allocates nothing checks its arguments before it touches a device
     assert B.grad_norm_static(0x1000, -1, None, 0, 1.0, 0x2000) == B.ERR_INVALID_ARG
     assert B.grad_norm_static(None, 8, None, 0, 1.0, 0x2000) == B.ERR_INVALID_ARG
@@ -118,13 +120,20 @@ def test_tuning_keys(B):
     with pytest.raises(B.RlxError):
         B.set_tuning("no_such_key", 1)
     assert B.get_tuning("no_such_key") == -1
-    for key, top in (("norm_pack", 3), ("convert_variant", 3), ("final_batch", 40)):
+    assert B.get_tuning("norm_fused") == 2 and B.get_tuning("norm_pack") == 3        # the shipped choices
+    assert B.get_tuning("norm_keep_mb") == 0 and B.get_tuning("update_reverse") == 0
+    for key, top in (("norm_pack", 3), ("convert_variant", 3), ("final_batch", 40), ("norm_fused", 1), ("norm_keep_mb", 4096),
+                     ("update_reverse", 1)):
         default = B.get_tuning(key)
         B.set_tuning(key, top)
         assert B.get_tuning(key) == top
         B.set_tuning(key, default)
     with pytest.raises(B.RlxError):
         B.set_tuning("convert_variant", 4)
+    with pytest.raises(B.RlxError):
+        B.set_tuning("norm_fused", 3)
+    with pytest.raises(B.RlxError):
+        B.set_tuning("norm_keep_mb", 4097)
     # every update variant has a kernel name; the default names the shipped tile shape
     names = [B.update_variant_name(v) for v in range(17)]
     assert all(names) and len(set(names)) == 17 and B.update_variant_name(17) == ""
