@@ -61,60 +61,69 @@ def cpu_baseline(O, host, sample, g_clip, hyper, step, seconds=5.0):
     """The oracle's threaded FP16 step on a slice of the same workload, on the host's cores: the update alone
     (the configuration of the headline), and norm + clip + update with the larger gradients of the clip
     configuration (FP64 sum of squares, sqrt, scale = max/(norm+1e-6f) iff norm > max, then the update with
-    the scaled and re-rounded gradients).  Each leg is repeated until about `seconds` of wall time have
-    passed, with 16 threads (the CPU share of a one-GPU box) and with every core the process may use."""
-    p, g, m, v = sample
+    the scaled and re-rounded gradients), with 16 threads (the CPU share of a one-GPU box) and with every core the
+    process may use.
+    Every timed pass starts from the saved state of step 99 (restored outside the timed region): the port's speed
+    depends on the values (this host's divider is data dependent), and repeating one step in place on fixed
+    gradients drives the first moments towards zero and the step from 12.4 to 4.9 ms per Mi parameters.  Each leg
+    is repeated until about `seconds` of wall time have passed."""
+    p0, g, m0, v0 = sample
     cpus = host_cpus()
     t16 = min(16, cpus["affinity"])
     t_all = cpus["affinity"]
     bc1, bc2 = host.bias_correction(hyper["beta1"], step), host.bias_correction(hyper["beta2"], step)
     args = (hyper["lr"], hyper["beta1"], hyper["beta2"], hyper["eps"], hyper["wd"], bc1, bc2)
 
-    def rate(arrays, max_norm, threads, budget):
-        O.step_fp16_threaded(None, *arrays, *args, max_norm, threads)          # touch pages, warm caches
-        reps, t0 = 0, time.perf_counter()
+    def rate(n, grad, max_norm, threads, budget):
+        """params/s over passes that each start from the saved state; (rate, passes, timed seconds)."""
+        p, m, v = p0[:n].copy(), m0[:n].copy(), v0[:n].copy()
+        gg = grad[:n]
+        O.step_fp16_threaded(None, p, gg, m, v, *args, max_norm, threads)        # touch pages, warm caches
+        reps, timed, wall0 = 0, 0.0, time.perf_counter()
         while True:
-            O.step_fp16_threaded(None, *arrays, *args, max_norm, threads)
+            p[:], m[:], v[:] = p0[:n], m0[:n], v0[:n]
+            t0 = time.perf_counter()
+            O.step_fp16_threaded(None, p, gg, m, v, *args, max_norm, threads)
+            timed += time.perf_counter() - t0
             reps += 1
-            el = time.perf_counter() - t0
-            if el >= budget or reps >= 200:
+            if time.perf_counter() - wall0 >= budget or reps >= 200:
                 break
-        return arrays[0].size * reps / el, reps, el
+        return n * reps / timed, reps, timed
 
+    n_all = p0.size
     out = {"unit": "params/s", "kind": "port", "nproc": cpus["nproc"], "affinity": cpus["affinity"],
            "cgroup_cpus": cpus["cgroup_cpus"], "threads": t16, "threads_all_cores": t_all}
-    upd, reps, el = rate((p, g, m, v), 0.0, t16, seconds)
+    upd, reps, el = rate(n_all, g, 0.0, t16, seconds)
     out["update"] = upd
     out["value"] = upd
     out["cores"] = t16
     out["gbps"] = BYTES_UPDATE * upd / 1e9
-    clip_arrays = (p.copy(), g_clip, m.copy(), v.copy())
-    out["norm_clip_update"], reps_c, el_c = rate(clip_arrays, 1.0, t16, seconds)
+    out["norm_clip_update"], reps_c, el_c = rate(n_all, g_clip, 1.0, t16, seconds)
     if t_all != t16:
-        out["update_all_cores"], _, _ = rate((p, g, m, v), 0.0, t_all, seconds * 0.6)
-        out["norm_clip_update_all_cores"], _, _ = rate(clip_arrays, 1.0, t_all, seconds * 0.6)
+        out["update_all_cores"], _, _ = rate(n_all, g, 0.0, t_all, seconds * 0.6)
+        out["norm_clip_update_all_cores"], _, _ = rate(n_all, g_clip, 1.0, t_all, seconds * 0.6)
     else:
         out["update_all_cores"], out["norm_clip_update_all_cores"] = out["update"], out["norm_clip_update"]
-    n1 = min(p.size, 4 * 1024 * 1024)                                # one thread, first 4 Mi parameters
-    out["single_thread"], _, _ = rate(tuple(a[:n1].copy() for a in (p, g, m, v)), 0.0, 1, 2.0)
+    n1 = min(n_all, 4 * 1024 * 1024)                                 # one thread, first 4 Mi parameters
+    out["single_thread"], _, _ = rate(n1, g, 0.0, 1, 2.0)
     out["single_thread_value"] = out["single_thread"]
     # the reference's own CPU-runnable case: one flat tensor of 1,048,576 parameters, full size (first Mi of the sample)
     n0 = 1 << 20
-    flat = tuple(a[:n0].copy() for a in (p, g, m, v))
-    r1, _, _ = rate(flat, 0.0, 1, 1.0)
-    r16, _, _ = rate(flat, 0.0, t16, 1.0)
+    r1, _, _ = rate(n0, g, 0.0, 1, 1.0)
+    r16, _, _ = rate(n0, g, 0.0, t16, 1.0)
     out["flat_1m_ms_per_step_one_thread"] = n0 / r1 * 1e3
     out["flat_1m_ms_per_step_threads"] = n0 / r16 * 1e3
-    out["sample"] = ("%d-param slice of embed_tokens (Qwen3-0.6B state after 99 steps), %d + %d repeated steps in %.1f + %.1f s; "
-                     "update leg: g of step 100; norm+clip+update leg: g~N(0,5e-3), max_norm 1.0; oracle's threaded AdamW "
-                     "loop, gcc -O3, no FMA contraction, static contiguous split over the threads"
-                     % (p.size, reps, reps_c, el, el_c))
+    out["sample"] = ("%d-param slice of embed_tokens (Qwen3-0.6B state after 99 steps), %d + %d passes of %.1f + %.1f s timed, "
+                     "each from the saved state; update leg: g of step 100; norm+clip+update leg: g~N(0,5e-3), max_norm 1.0; "
+                     "oracle's threaded AdamW loop, gcc -O3, no FMA contraction, static contiguous split over the threads"
+                     % (n_all, reps, reps_c, el, el_c))
     return out
 
 
 class HostList:
     """Host copies of the first `count` tensors of a ParamStore whose tensors are all FP16 (weights, gradients,
-    moments as the pools hold them, padding between tensors included), for the CPU legs at full size."""
+    moments as the pools hold them, padding between tensors included), for the CPU legs at full size; and a
+    second copy of weights and moments, from which every timed pass starts."""
 
     def __init__(self, st, count):
         import numpy as np
@@ -127,8 +136,12 @@ class HostList:
         half = lambda t, n: t[:n].view(torch.int16).cpu().numpy().view(np.uint16)
         self.p, self.g = half(st.p16, end_pg), half(st.g16, end_pg)
         self.m, self.v = st.m[:end].cpu().numpy(), st.v[:end].cpu().numpy()
+        self.saved = (self.p.copy(), self.m.copy(), self.v.copy())
         self.params = sum(self.sizes)
         self.end_pg = end_pg
+
+    def restore(self):
+        self.p[:], self.m[:], self.v[:] = self.saved
 
     def gradients(self, st):
         """The store's present gradients of the same tensors (another leg's gradients)."""
@@ -137,33 +150,56 @@ class HostList:
         return st.g16[:self.end_pg].view(torch.int16).cpu().numpy().view(np.uint16)
 
 
-def cpu_list_legs(O, host, hl, hyper, step, threads, g_clip=None, per_tensor=False, budget=4.0):
+def cpu_list_legs(O, host, hl, hyper, step, threads, g_clip=None, per_tensor=False, budget=4.0, single_thread=True):
     """The oracle's threaded step over the whole tensor list held in `hl`, timed on the host: the update alone,
-    optionally norm + clip + update with the gradients g_clip, optionally the update as one call per tensor.
-    Each leg: one untimed pass, then repeated until `budget` seconds or 20 passes."""
+    optionally norm + clip + update with the gradients g_clip, optionally the update as one call per tensor, and
+    the same legs on ONE thread.  Every timed pass starts from the saved state (restored outside the timed
+    region; the port's speed depends on the values, see cpu_baseline).  Each leg: one untimed pass, then passes
+    until `budget` seconds of wall time or 20 of them; a pass that takes more than half a second is timed once."""
     bc1, bc2 = host.bias_correction(hyper["beta1"], step), host.bias_correction(hyper["beta2"], step)
     args = (hyper["lr"], hyper["beta1"], hyper["beta2"], hyper["eps"], hyper["wd"], bc1, bc2)
+    pools = (hl.off_pg, hl.off, hl.sizes)
+    ptr_g = O.list_pointers(hl.p, hl.g, hl.m, hl.v, *pools)
+    ptr_c = O.list_pointers(hl.p, g_clip, hl.m, hl.v, *pools) if g_clip is not None else None
 
-    def timed(fn):
-        fn()
-        reps, t0 = 0, time.perf_counter()
-        while True:
+    def timed(fn, warm=True):
+        if warm:
             fn()
+        reps, total, wall0 = 0, 0.0, time.perf_counter()
+        while True:
+            hl.restore()
+            t0 = time.perf_counter()
+            fn()
+            dt = time.perf_counter() - t0
+            total += dt
             reps += 1
-            el = time.perf_counter() - t0
-            if el >= budget or reps >= 20:
-                return el / reps * 1e3, reps
+            if dt > 0.5 or time.perf_counter() - wall0 >= budget or reps >= 20:
+                return total / reps * 1e3, reps
+
+    def update(th):
+        return lambda: O.step_list_fp16_threaded(hl.p, hl.g, hl.m, hl.v, *pools, *args, 0.0, th, pointers=ptr_g)
+
+    def clip(th):
+        return lambda: O.step_list_fp16_threaded(hl.p, g_clip, hl.m, hl.v, *pools, *args, 1.0, th, pointers=ptr_c)
 
     out = {"params": hl.params, "tensors": hl.count, "threads": threads}
-    ms, reps = timed(lambda: O.step_list_fp16_threaded(hl.p, hl.g, hl.m, hl.v, hl.off_pg, hl.off, hl.sizes, *args, 0.0, threads))
+    ms, reps = timed(update(threads))
     out.update(update_ms=ms, update_params_per_s=hl.params / (ms * 1e-3), update_gbps=BYTES_UPDATE * hl.params / (ms * 1e-3) / 1e9,
                update_passes=reps)
     if g_clip is not None:
-        ms, reps = timed(lambda: O.step_list_fp16_threaded(hl.p, g_clip, hl.m, hl.v, hl.off_pg, hl.off, hl.sizes, *args, 1.0, threads))
+        ms, reps = timed(clip(threads))
         out.update(norm_clip_update_ms=ms, norm_clip_update_params_per_s=hl.params / (ms * 1e-3), norm_clip_update_passes=reps)
     if per_tensor:
-        ms, reps = timed(lambda: O.update_per_tensor_fp16_threaded(hl.p, hl.g, hl.m, hl.v, hl.off_pg, hl.off, hl.sizes, *args, threads))
+        ms, reps = timed(lambda: O.update_per_tensor_fp16_threaded(hl.p, hl.g, hl.m, hl.v, *pools, *args, threads, pointers=ptr_g))
         out.update(per_tensor_loop_update_ms=ms, per_tensor_loop_passes=reps)
+    if single_thread:
+        big = hl.params > (1 << 26)              # a pass takes seconds: no warm-up pass
+        ms, _ = timed(update(1), warm=not big)
+        out.update(single_thread_update_ms=ms, single_thread_update_params_per_s=hl.params / (ms * 1e-3))
+        if g_clip is not None:
+            ms, _ = timed(clip(1), warm=not big)
+            out.update(single_thread_norm_clip_update_ms=ms)
+    hl.restore()
     return out
 
 
@@ -238,16 +274,8 @@ def measure_workload(name, pkg, host, steps, warmup, chunk=0, O=None):
     opt.step_ = 999
     stream = torch.cuda.current_stream().cuda_stream
     bpp = 28 if master else BYTES_UPDATE
-    upd = time_events(lambda: opt.step(), warmup, steps)
-    nrm = time_events(lambda: opt.plan.grad_norm(1.0, stream), warmup, steps)
-
-    def clip_step():
-        opt.plan.grad_norm(1.0, stream)
-        opt.step(fused_clip=True)
-
-    both = time_events(clip_step, warmup, steps)
-    norm, scale, _ = opt.plan.norm_read(stream)
-    graph_ms = graph_clip_step_ms(opt, B, warmup, steps) if name != "qwen3-8b" else None
+    # the CPU legs first, on host copies of the seeded state as it is now: the timed GPU steps below repeat one step on
+    # the same gradients and move the state on, and the CPU port's speed depends on the values
     cpu = None
     if O is not None and not master:
         hyper = dict(lr=1e-5, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01)
@@ -259,7 +287,7 @@ def measure_workload(name, pkg, host, steps, warmup, chunk=0, O=None):
                 tot += specs[count].n
                 count += 1
             hl = HostList(st, count)
-            cpu = cpu_list_legs(O, host, hl, hyper, 1000, t16, g_clip=hl.g, budget=4.0)
+            cpu = cpu_list_legs(O, host, hl, hyper, 1000, t16, g_clip=hl.g, budget=4.0, single_thread=False)
             cpu["sample"] = "the first %d tensors of the list (%d parameters); full-size figures extrapolated by parameter count" % (count, tot)
             for key in ("update_ms", "norm_clip_update_ms"):
                 cpu["extrapolated_full_" + key] = cpu[key] * N / tot
@@ -268,6 +296,16 @@ def measure_workload(name, pkg, host, steps, warmup, chunk=0, O=None):
             cpu = cpu_list_legs(O, host, hl, hyper, 1000, t16, g_clip=hl.g, per_tensor=(name == "ragged"), budget=2.0)
             cpu["sample"] = "the whole configuration"
         del hl
+    upd = time_events(lambda: opt.step(), warmup, steps)
+    nrm = time_events(lambda: opt.plan.grad_norm(1.0, stream), warmup, steps)
+
+    def clip_step():
+        opt.plan.grad_norm(1.0, stream)
+        opt.step(fused_clip=True)
+
+    both = time_events(clip_step, warmup, steps)
+    norm, scale, _ = opt.plan.norm_read(stream)
+    graph_ms = graph_clip_step_ms(opt, B, warmup, steps) if name != "qwen3-8b" else None
     scale_ms = time_events(lambda: opt.plan.scale_grads(stream), 1, 5)   # shrinks the gradients: last leg
     out = {
         "workload": what, "params": N, "tensors": len(specs), "bytes_per_param": bpp,
@@ -287,8 +325,18 @@ def measure_workload(name, pkg, host, steps, warmup, chunk=0, O=None):
         flat = host.ParamStore([L.TensorSpec("flat", N, L.DTYPE_F16, 0, 0)], "cuda:0")
         flat.fill("p", SEED_P, 1.0, p_std)
         flat.fill("g", SEED_G, 0.0, g_std)
+        flat.fill("m", SEED_P + 1, 0.0, 1e-4)
+        flat.fill("v", SEED_P + 2, 1e-8, 1e-8, flags=B.FILL_ABS)
         fopt = host.AdamWOptimizer(flat, lr=1e-5)
         fopt.step_ = 999
+        if O is not None:      # the same element count as one flat tensor on the host
+            hl = HostList(flat, 1)
+            fcpu = cpu_list_legs(O, host, hl, dict(lr=1e-5, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01), 1000,
+                                 min(16, host_cpus()["affinity"]), budget=2.0)
+            out["cpu"]["flat_update_ms"] = fcpu["update_ms"]
+            out["cpu"]["update_vs_flat"] = out["cpu"]["update_ms"] / fcpu["update_ms"]
+            out["cpu"]["per_tensor_loop_vs_flat"] = out["cpu"]["per_tensor_loop_update_ms"] / fcpu["update_ms"]
+            del hl
         out["flat_update_ms"] = time_events(lambda: fopt.step(), warmup, steps)
         out["flat_norm_ms"] = time_events(lambda: fopt.plan.grad_norm(1.0, stream), warmup, steps)
 
@@ -302,14 +350,6 @@ def measure_workload(name, pkg, host, steps, warmup, chunk=0, O=None):
         out["clip_step_vs_flat"] = both / out["flat_clip_step_ms"]
         out["flat_graph_clip_step_ms"] = graph_clip_step_ms(fopt, B, warmup, steps)
         out["graph_clip_step_vs_flat"] = graph_ms / out["flat_graph_clip_step_ms"]
-        if O is not None:      # the same element count as one flat tensor on the host
-            hl = HostList(flat, 1)
-            fcpu = cpu_list_legs(O, host, hl, dict(lr=1e-5, beta1=0.9, beta2=0.999, eps=1e-8, wd=0.01), 1000,
-                                 min(16, host_cpus()["affinity"]), budget=2.0)
-            out["cpu"]["flat_update_ms"] = fcpu["update_ms"]
-            out["cpu"]["update_vs_flat"] = out["cpu"]["update_ms"] / fcpu["update_ms"]
-            out["cpu"]["per_tensor_loop_vs_flat"] = out["cpu"]["per_tensor_loop_update_ms"] / fcpu["update_ms"]
-            del hl
         del fopt, flat
     return out
 
@@ -420,6 +460,13 @@ def main():
     # gradients of the measured step (step 100)
     st.fill("g", SEED_G + 100, 0.0, 1e-4, zero_row_frac=0.9, only=("embed_tokens",))
 
+    # ---- CPU baseline inputs: the state after exactly 99 steps and the gradients of step 100, taken BEFORE the timed
+    # GPU steps (which repeat step 100 on the same gradients and so move the state on: the CPU port's speed depends on
+    # the values, the GPU kernel's does not).  A slice of the embedding, and the whole configuration (7.2 GB). ----
+    n_s = 32 * 1024 * 1024
+    sample = None if args.no_cpu else tuple(grab(k, emb, 0, n_s) for k in ("p", "g", "m", "v"))
+    host_list = None if args.no_cpu else HostList(st, len(specs))
+
     # ---- timed: update only (configs[1]) ----
     def run(fn, warmup, steps):
         """W untimed steps, then exactly `steps` launches back to back between two HIP events on the
@@ -452,11 +499,6 @@ def main():
     kernel_ms = ev_ms
     achieved = BYTES_UPDATE * N / (kernel_ms * 1e-3) / 1e9
 
-    # ---- CPU baseline sample: state of the headline configuration (before the clip leg moves it on) ----
-    n_s = 32 * 1024 * 1024
-    sample = None if args.no_cpu else tuple(grab(k, emb, 0, n_s) for k in ("p", "g", "m", "v"))
-    # the whole configuration on the host, for the full-size CPU legs (7.2 GB)
-    host_list = None if args.no_cpu else HostList(st, len(specs))
 
     # ---- timed: norm + clip scale + fused update (configs[2]); larger gradients so that clipping is active ----
     st.fill("g", SEED_G + 1000, 0.0, 5e-3)

@@ -216,7 +216,10 @@ def step_fp16_threaded(master, model, grad, m, v, lr, beta1, beta2, eps, wd, bc1
                                             max_norm, threads))
 
 
-def _list_pointers(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts):
+def list_pointers(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts):
+    """The pointer arrays of a tensor list inside four pools (FP16 weights and gradients share the offsets off_pg,
+    FP32 moments the offsets off_state; counts[i] elements each), built once for repeated calls.  The pools must
+    stay alive and in place while the result is used."""
     k = len(counts)
     ptr = C.c_void_p * k
     cnt = (C.c_int64 * k)(*[int(c) for c in counts])
@@ -228,17 +231,17 @@ def _list_pointers(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts):
 
 
 def step_list_fp16_threaded(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts, lr, beta1, beta2, eps, wd,
-                            bc1, bc2, max_norm, threads):
-    """Norm (if max_norm > 0) + clip + update of a LIST of FP16 tensors that live inside four pools (FP16 weights
-    and gradients share the offsets off_pg, FP32 moments the offsets off_state; counts[i] elements each), with
-    the concatenated index space split over `threads` host threads.  In place.  Returns the pre-clip norm."""
-    k, model, grad, m, v, cnt = _list_pointers(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts)
+                            bc1, bc2, max_norm, threads, pointers=None):
+    """Norm (if max_norm > 0) + clip + update of a LIST of FP16 tensors that live inside four pools, with the
+    concatenated index space split over `threads` host threads.  In place.  Returns the pre-clip norm.
+    `pointers`: the result of list_pointers for these pools (saves building it on every call)."""
+    k, model, grad, m, v, cnt = pointers or list_pointers(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts)
     return float(lib.orc_step_list_fp16_threaded(k, model, grad, m, v, cnt, lr, beta1, beta2, eps, wd, bc1, bc2,
                                                  max_norm, threads))
 
 
 def update_per_tensor_fp16_threaded(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts, lr, beta1, beta2, eps,
-                                    wd, bc1, bc2, threads):
+                                    wd, bc1, bc2, threads, pointers=None):
     """The same update as a loop over the tensors, each split over the threads by itself."""
-    k, model, grad, m, v, cnt = _list_pointers(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts)
+    k, model, grad, m, v, cnt = pointers or list_pointers(p_pool, g_pool, m_pool, v_pool, off_pg, off_state, counts)
     lib.orc_update_per_tensor_fp16_threaded(k, model, grad, m, v, cnt, lr, beta1, beta2, eps, wd, bc1, bc2, threads)
