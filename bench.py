@@ -14,7 +14,15 @@ update, norm, norm + fused-clip update, each in ms and GB/s (seeded state, no or
 hold the parity of these configurations).  --configs none skips them (short profiler runs).
 
 Prints ONE JSON line.  The CPU oracle is used here only as the checker of a sample and as the
-timed CPU baseline.
+timed CPU baseline: the oracle's threaded step on a slice of the embedding's state ("cpu_baseline") and on every
+configuration at its own size ("cpu_baseline.configs": all 310 tensors of Qwen3-0.6B, the flat tensor, the 4,096-tensor
+list as one split / as a loop of one call per tensor / beside one flat tensor, a 1e9-parameter slice of Qwen3-8B),
+with 16 threads and with one; its inputs are copied to the host before the timed GPU steps and every CPU pass starts
+from that saved state.
+
+Beside the eager legs, "clip_step" holds the parts of the clip step in the same run (plain update on dense gradients,
+fused-clip update alone, norm) and every configuration holds "graph_clip_step_ms": norm + scheduled fused-clip update
+recorded once as a HIP graph and replayed.
 
 --workload selects one of the other configurations as the line's subject instead (flat-1m,
 qwen3-0.6b-master, ragged, qwen3-8b): the same kind of line with fewer legs.
