@@ -152,9 +152,9 @@ int64_t rlx_plan_chunk_elems(const rlx_plan* plan);
  * in a fixed order, so that the result is the same bits on every run.  That last sum is a
  * second launch, or, for launches of up to 256 workgroups, the tail of the first one: the
  * workgroup that finishes last (found by counting tickets, which decides who adds but not in
- * which order) does it.  Both forms give the same bits ("norm_fused" below chooses).  The tickets live in the
- * plan and are zero between launches: norm launches of ONE plan must not overlap (two streams, two threads),
- * or the counters can be left non-zero and later norms of that plan never complete their sum.  Writes
+ * which order) does it.  Both forms give the same bits ("norm_fused" below chooses).  Partials and tickets live
+ * in the plan: norm launches of ONE plan must not overlap (two streams, two threads); launches that do spoil each
+ * other's result, not those of later launches (the ticket counters only count up and need no reset).  Writes
  * {sum_sq, norm = sqrtf((float)sum_sq), scale} to the plan's device result, where
  * scale = max_norm / (norm + 1e-6f) iff norm > max_norm, else 1.0f (a NaN norm gives
  * 1.0f, as the reference's comparison does; max_norm = INFINITY measures without clipping).
@@ -190,7 +190,8 @@ const double* rlx_plan_partials_device_ptr(const rlx_plan* plan);
  * GPU share the array: calls that overlap on one GPU (two streams, two threads) race; calls on one stream
  * do not.  Nothing in the array has to start at zero: every call writes each slot that it later reads (this
  * entry point always adds the partials in a second launch, whatever "norm_fused" says: the one-launch form keeps
- * counters that must be zero between calls, which overlapping calls on a shared array could spoil for good).
+ * counters that are only valid from call to call while the number of workgroups stays the same, and calls of any
+ * size share this array).
  */
 int rlx_grad_norm_static(const uint16_t* half_grads, int64_t n_half, const float* float_grads, int64_t n_float,
                          int64_t chunk_elems, float max_norm, void* result_dev, void* stream);

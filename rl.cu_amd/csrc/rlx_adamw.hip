@@ -44,8 +44,9 @@
 // library's device image (2.1 MiB on every GPU the library runs on, until the process ends).  Layout, in
 // doubles: [0, 2^18) per-chunk FP64 partials; [2^18, 2^18 + 2^14) group partials (one per 16 chunks, used with
 // 512-element chunks).  Nothing in it has to start at zero: every call writes each slot that it later reads (the
-// entry point always adds the partials in a second launch; the one-launch form needs counters that must be zero
-// between calls, and calls that overlap on this shared array could leave them otherwise for good).  The name
+// entry point always adds the partials in a second launch; the one-launch form needs counters that stay valid
+// from call to call only while the number of workgroups stays the same, and calls of any size share this array).
+// The name
 // stands for the array only in device code; host code uses the address that hipGetSymbolAddress returns for the
 // current device (static_scratch below), never the name.
 constexpr int64_t kStaticMaxPartials = 1 << 18;
@@ -587,7 +588,7 @@ __global__ __launch_bounds__(BLOCK) void adamw_chunk_kernel(
 
 constexpr int kGroupChunks = 16;              // 512-element chunks per group partial
 constexpr int kTicketGroup = 64;              // workgroups per first-level ticket counter
-constexpr int kTicketStride = 32;             // 32-bit words from one counter to the next (128 bytes: a line each)
+constexpr int kTicketStride = 16;             // 64-bit words from one counter to the next (128 bytes: a line each)
 constexpr int64_t kMaxFusedWgs = 8192;        // largest grid whose last workgroup adds the partials itself
 constexpr int64_t kTicketWords = (kMaxFusedWgs / kTicketGroup + 1) * kTicketStride;
 static_assert(kStaticMaxGroups * kGroupChunks == kStaticMaxPartials, "the static scratch holds the partials and their groups");
@@ -598,8 +599,9 @@ struct NormTail {
     int64_t n_values;
     float max_norm;
     NormResult* out;
-    uint32_t* tickets;           // [0]: second-level counter; [(1 + g) * kTicketStride]: counter of workgroups
-                                 // 64g .. 64g+63.  All zero between launches.
+    uint64_t* tickets;           // [0]: second-level counter; [(1 + g) * kTicketStride]: counter of workgroups
+                                 // 64g .. 64g+63.  Never reset: every launch of the same grid adds the same
+                                 // amount to each counter, and "last" is a ticket that completes a multiple of it.
     int64_t plain_below;         // > 0: the launch walks the chunks from the last to the first, and chunks with an
                                  // index below this are read with ordinary instead of non-temporal loads, so that
                                  // what the norm reads last, the start of the gradients, is what stays in the
@@ -669,13 +671,17 @@ __device__ __forceinline__ void publish(double* slot, double x) {
 // final sum reads must have been stored with publish() by lanes of the workgroup's first wavefront before the call.
 // Two levels of counters (64 workgroups share a first-level counter, the last of each 64 takes a second-level
 // ticket), so that thousands of workgroups finishing together do not queue on one address (one counter for
-// all: 12 ns per workgroup, 100 us for 8,192).  Whoever draws a counter's last ticket puts the counter back to
-// zero for the next launch.
+// all: 12 ns per workgroup, 100 us for 8,192).
+// The counters only ever count up (64 bits: they do not wrap): a launch of G workgroups adds the size of group g
+// to counter g and the number of groups to the second-level counter, so as long as every launch on these counters
+// has the same G (the host clears them when G changes), the ticket that completes a multiple of that amount is
+// the launch's last.  Nothing has to be put back to zero, a recorded launch replays as it is, and two launches that
+// overlap by mistake spoil each other's result but leave the counters at a multiple again for the launches after.
 // Ordering: the published values are device-scope stores, the wavefront waits until they have been acknowledged
 // and only then takes its ticket; the last workgroup reads them with device-scope loads after its ticket has
 // come back.  A full device-scope fence in front of the ticket would do as well, but it writes the whole L2 back
 // and measured 67 ns per workgroup, one after the other across the device (550 us for 8,192 workgroups).
-__device__ __forceinline__ bool last_workgroup(uint32_t* tickets, int* lds_flag) {
+__device__ __forceinline__ bool last_workgroup(uint64_t* tickets, int* lds_flag) {
     if (threadIdx.x < 64) {
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         wait_for_memory();                  // this wavefront's published values have arrived before its ticket is taken
@@ -683,14 +689,12 @@ __device__ __forceinline__ bool last_workgroup(uint32_t* tickets, int* lds_flag)
             const uint32_t n_wg = gridDim.x, grp = blockIdx.x / kTicketGroup;
             const uint32_t n_grp = (n_wg + kTicketGroup - 1) / kTicketGroup;
             const uint32_t in_grp = grp + 1 < n_grp ? (uint32_t)kTicketGroup : n_wg - grp * kTicketGroup;
-            uint32_t* c1 = tickets + (size_t)(1 + grp) * kTicketStride;
+            uint64_t* c1 = tickets + (size_t)(1 + grp) * kTicketStride;
             int last = 0;
-            if (__hip_atomic_fetch_add(c1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == in_grp - 1) {
-                __hip_atomic_store(c1, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                if (__hip_atomic_fetch_add(tickets, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == n_grp - 1) {
-                    __hip_atomic_store(tickets, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-                    last = 1;
-                }
+            const uint64_t t1 = __hip_atomic_fetch_add(c1, (uint64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+            if (t1 % in_grp == 0) {
+                const uint64_t t0 = __hip_atomic_fetch_add(tickets, (uint64_t)1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) + 1;
+                last = t0 % n_grp == 0;
             }
             *lds_flag = last;
         }
@@ -1525,8 +1529,9 @@ struct rlx_plan {
     std::vector<std::pair<void*, int64_t>> idle_grads;
     bool idle_by_range;
     double* d_partials;      // one allocation: per-chunk partials, then the group partials (one per 16 chunks),
-    double* d_groups;        // then the ticket counters of the norm launch (zero between launches)
-    uint32_t* d_tickets;
+    double* d_groups;        // then the ticket counters of the one-launch norm
+    uint64_t* d_tickets;
+    int64_t ticket_grid;     // workgroups of the last one-launch norm on these counters (0: none yet)
     NormResult* d_norm;
     NormResult* h_norm;      // pinned
     // host-free replay: a table of per-step hyper-parameters on the device, the entry that the next scheduled
@@ -1588,7 +1593,8 @@ struct NormWork {
     int64_t n_chunks, chunk_elems;
     double* partials;            // one per chunk
     double* groups;              // one per 16 chunks; only used with 512-element chunks
-    uint32_t* tickets;           // kTicketWords words, all zero between launches; null: never the one-launch form
+    uint64_t* tickets;           // kTicketWords 64-bit counters; null: never the one-launch form
+    int64_t* ticket_grid;        // workgroups of the last one-launch norm on these counters
     NormResult* result;
 };
 
@@ -1646,11 +1652,19 @@ int launch_norm_nt(const NormWork& w, float max_norm, hipStream_t s) {
     };
     bool fused = false;
     hipError_t e = hipSuccess;
+    // the counters hold multiples of what one launch of the previous grid added: another grid starts from zero
+    const auto same_grid = [&](int64_t grid) -> hipError_t {
+        if (*w.ticket_grid == grid) return hipSuccess;
+        *w.ticket_grid = grid;
+        return clear_range(w.tickets, (int64_t)(sizeof(uint64_t) * kTicketWords), s);
+    };
     if (!grouped) {
         int64_t g = norm_grid > 0 ? norm_grid : w.n_chunks;
         if (g > w.n_chunks) g = w.n_chunks;
         if (g > kMaxNormGrid) g = kMaxNormGrid;
         fused = want_fused(g);
+        if (fused) e = same_grid(g);
+        if (e != hipSuccess) return hip_fail(e, "norm ticket counters");
         if (lanes >= 512) e = launch_partials<NT, POOLS, 512>(w, g, fused, tail, s);
         else if (lanes == 256) e = launch_partials<NT, POOLS, 256>(w, g, fused, tail, s);
         else e = launch_partials<NT, POOLS, 128>(w, g, fused, tail, s);
@@ -1680,6 +1694,8 @@ int launch_norm_nt(const NormWork& w, float max_norm, hipStream_t s) {
         const int64_t g = (w.n_chunks + per_wg - 1) / per_wg;
         if (g > kMaxNormGrid) return RLX_ERR_TOO_LARGE;
         fused = want_fused(g);
+        if (fused) e = same_grid(g);
+        if (e != hipSuccess) return hip_fail(e, "norm ticket counters");
         if (norm_pack == 3) e = launch_small_chunks<NT, POOLS, 8, 2>(w, g, fused, tail, s);
         else e = launch_small_chunks<NT, POOLS, 8, 4>(w, g, fused, tail, s);
     }
@@ -1870,17 +1886,17 @@ int rlx_plan_create(const rlx_tensor_desc* descs, int64_t count, int64_t chunk_e
                 p->idle_by_range = false;
         }
     }
-    p->d_recs = nullptr; p->d_active = nullptr; p->n_active = 0; p->d_partials = nullptr; p->d_groups = nullptr; p->d_tickets = nullptr; p->d_norm = nullptr; p->h_norm = nullptr;
+    p->d_recs = nullptr; p->d_active = nullptr; p->n_active = 0; p->d_partials = nullptr; p->d_groups = nullptr; p->d_tickets = nullptr; p->ticket_grid = 0; p->d_norm = nullptr; p->h_norm = nullptr;
     p->d_sched = nullptr; p->sched_cap = 0; p->sched_len = 0; p->d_header = nullptr;
 
     hipError_t e = hipGetDevice(&p->device);
     if (e == hipSuccess) e = hipMalloc((void**)&p->d_recs, sizeof(ChunkRec) * (size_t)n_chunks);
     const size_t n_sums = (size_t)n_chunks + (size_t)norm_groups(n_chunks);
-    if (e == hipSuccess) e = hipMalloc((void**)&p->d_partials, sizeof(double) * n_sums + sizeof(uint32_t) * (size_t)kTicketWords);
+    if (e == hipSuccess) e = hipMalloc((void**)&p->d_partials, sizeof(double) * n_sums + sizeof(uint64_t) * (size_t)kTicketWords);
     if (e == hipSuccess) {
         p->d_groups = p->d_partials + n_chunks;
-        p->d_tickets = (uint32_t*)(p->d_partials + n_sums);
-        e = hipMemset(p->d_tickets, 0, sizeof(uint32_t) * (size_t)kTicketWords);
+        p->d_tickets = (uint64_t*)(p->d_partials + n_sums);
+        e = hipMemset(p->d_tickets, 0, sizeof(uint64_t) * (size_t)kTicketWords);
     }
     if (e == hipSuccess) e = hipMalloc((void**)&p->d_norm, sizeof(NormResult));
     if (e == hipSuccess) e = hipHostMalloc((void**)&p->h_norm, sizeof(NormResult), hipHostMallocDefault);
@@ -1943,7 +1959,8 @@ int rlx_plan_grad_norm(rlx_plan* p, float max_norm, void* stream) {
     NormWork w;
     memset(&w, 0, sizeof(w));
     w.recs = p->d_recs; w.n_chunks = p->n_chunks; w.chunk_elems = p->chunk_elems;
-    w.partials = p->d_partials; w.groups = p->d_groups; w.tickets = p->d_tickets; w.result = p->d_norm;
+    w.partials = p->d_partials; w.groups = p->d_groups; w.tickets = p->d_tickets; w.ticket_grid = &p->ticket_grid;
+    w.result = p->d_norm;
     return launch_norm<false>(w, max_norm, (hipStream_t)stream);
 }
 
@@ -1996,7 +2013,7 @@ int rlx_grad_norm_static(const uint16_t* half_grads, int64_t n_half, const float
     memset(&w, 0, sizeof(w));
     w.pools = pp; w.n_chunks = n_chunks; w.chunk_elems = chunk_elems;
     w.partials = base; w.groups = base + kStaticMaxPartials;
-    w.tickets = nullptr;
+    w.tickets = nullptr; w.ticket_grid = nullptr;
     w.result = (NormResult*)result_dev;
     return launch_norm<true>(w, max_norm, (hipStream_t)stream);
 }
