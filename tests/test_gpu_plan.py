@@ -655,6 +655,8 @@ def test_packed_norm_pass_gives_the_same_partials(O, L, host, B, torch_gpu):
     (2048, [2048 * 200 + 3, 100]),                               # 256-lane workgroups
     (8192, [8192 * 4100 + 77, 9000]),                            # 4,103 workgroups: beyond the automatic limit
     (8192, [1]),                                                 # a single workgroup is its own last one
+    (1024, [1024 * 8192]),                                       # 8,192 workgroups: the largest one-launch grid
+    (1024, [1024 * 8192 + 1]),                                   # 8,193: one more, always a second launch
 ])
 def test_norm_summed_by_the_last_workgroup_equals_the_second_launch(O, B, torch_gpu, chunk, sizes):
     """The fixed-order sum of the partials as the tail of the first launch (the workgroup that draws the last
