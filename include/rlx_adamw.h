@@ -270,7 +270,8 @@ int rlx_plan_schedule_overrun(rlx_plan* plan, int64_t* overrun, void* stream);
  *                              CUs striding over the tiles, 12 = that with one workgroup walking a chunk
  *                              (10-12 with ordinary loads and stores; 13, 14 = 12, 11 with the shipped
  *                              kernel's non-temporal loads and system-scope non-temporal stores);
- *                              15, 16 = the shipped accesses with two / four 256-element sub-tiles per workgroup
+ *                              15, 16 = the shipped accesses with two / four 256-element sub-tiles per workgroup;
+ *                              17 = the shipped tile with lane pairs sharing 128-bit accesses
  *   "norm_grid"       0 = one workgroup per chunk, >0 = that many persistent workgroups
  *   "norm_nt"         1 = non-temporal loads in the norm pass (default), 0 = plain
  *   "norm_pack"       512-element chunks per workgroup in the norm pass: 0 = one, 1 = eight (one per

@@ -289,6 +289,56 @@ __device__ __forceinline__ void update_scalar32(const ChunkRec& r, int64_t i, co
 }
 
 // ---------------------------------------------------------------------------------------
+// The update of a whole, aligned tile of an FP16 tensor without master copy, two elements per lane as in update_tile,
+// but with half the memory instructions: the two lanes of a pair (2k, 2k+1) work on four consecutive elements, the
+// even lane loads the four first moments (128 bits) and the four gradients (64 bits), the odd lane the four second
+// moments and the four weights, each hands the other the half it needs (a swap inside the quad, no LDS), and the
+// results go back the same way: even lanes store four first moments, odd lanes four second moments and four weights.
+// One instruction then serves two streams, each half of the wavefront contiguous.  Same arithmetic per element.
+// ---------------------------------------------------------------------------------------
+
+template <int LANES, int SP, bool NTL, bool CLIP>
+__device__ __forceinline__ void update_tile_paired(const ChunkRec& r, int64_t off, int lane, Hyper h,
+                                                   const rlx_step_params* __restrict__ dev_params,
+                                                   const NormResult* __restrict__ norm)
+{
+    if (dev_params) {
+        h.lr = dev_params->lr; h.beta1 = dev_params->beta1; h.beta2 = dev_params->beta2; h.eps = dev_params->eps;
+        h.weight_decay = dev_params->weight_decay;
+        h.bc1_inv = 1.0f / dev_params->bias_correction1;
+        h.bc2_inv = 1.0f / dev_params->bias_correction2;
+    }
+    float scale = 1.0f;
+    if constexpr (CLIP) scale = norm->scale;
+    const float wd = (r.flags & RLX_TENSOR_NO_DECAY) ? 0.0f : h.weight_decay;
+    const bool odd = (lane & 1) != 0;
+    const int64_t pair = off + (int64_t)(lane & ~1) * 2;          // first of the pair's four elements
+    uint16_t* const p16 = (uint16_t*)r.p;
+    const f32x4 f = ldg<NTL>((const f32x4*)((odd ? r.v : r.m) + pair));
+    const u32x2 hw = ldg<NTL>((const u32x2*)((odd ? (const uint16_t*)p16 : (const uint16_t*)r.g) + pair));
+    // the even lane works on elements 0, 1 of the pair and needs v[0..1], p[0..1]; the odd lane on 2, 3 and needs
+    // m[2..3], g[2..3]
+    const float rf0 = __shfl_xor(odd ? f[0] : f[2], 1, 64), rf1 = __shfl_xor(odd ? f[1] : f[3], 1, 64);
+    const uint32_t rh = __shfl_xor(odd ? hw[0] : hw[1], 1, 64);
+    float g[2], m[2], v[2], w[2];
+    const uint32_t gbits = odd ? rh : hw[0], wbits = odd ? hw[1] : rh;
+    g[0] = h2f(gbits & 0xFFFFu); g[1] = h2f(gbits >> 16);
+    w[0] = h2f(wbits & 0xFFFFu); w[1] = h2f(wbits >> 16);
+    m[0] = odd ? rf0 : f[0]; m[1] = odd ? rf1 : f[1];
+    v[0] = odd ? f[2] : rf0; v[1] = odd ? f[3] : rf1;
+    if constexpr (CLIP) { g[0] = clip_f16(g[0], scale); g[1] = clip_f16(g[1], scale); }
+    adamw_elem(g[0], m[0], v[0], w[0], h, wd);
+    adamw_elem(g[1], m[1], v[1], w[1], h, wd);
+    // the even lane stores the pair's first moments, the odd lane its second moments and its weights
+    const float x0 = __shfl_xor(odd ? m[0] : v[0], 1, 64), x1 = __shfl_xor(odd ? m[1] : v[1], 1, 64);
+    const f32x4 out = odd ? f32x4{x0, x1, v[0], v[1]} : f32x4{m[0], m[1], x0, x1};
+    st_stream<SP>((f32x4*)((odd ? r.v : r.m) + pair), out);
+    const uint32_t mine = f2h(w[0]) | (f2h(w[1]) << 16);
+    const uint32_t other = __shfl_xor(mine, 1, 64);
+    if (odd) st_stream<SP>((u32x2*)(p16 + pair), u32x2{other, mine});
+}
+
+// ---------------------------------------------------------------------------------------
 // Update of one tile: E elements per lane, LANES lanes, TILE = E * LANES elements starting `off` elements into
 // the chunk `r`, of which `left` remain to the end of the chunk / tensor.  `lane` is this lane's index in the tile.
 // SP: 1 = system-scope non-temporal stores, 0 = non-temporal stores, 2 = ordinary stores; NTL: non-temporal loads.
@@ -308,6 +358,15 @@ __device__ __forceinline__ void update_tile(const ChunkRec& r, int64_t off, int6
     const int n_here = left < TILE ? (int)left : TILE;
     const bool is_f32 = (r.flags & kF32) != 0;
     const int valign = (r.flags >> kValignShift) & 0xF;
+    if constexpr (PH == 2 && E == 2) {
+        // whole tiles of plain FP16 tensors whose streams are aligned for a pair's 128-bit accesses; everything
+        // else (tails, FP32 tensors, master copy, gradient clearing, frozen and grad-only chunks) as below
+        if (left >= TILE && valign >= 4 && r.master == nullptr &&
+            !(r.flags & (kF32 | RLX_TENSOR_GRAD_ONLY | RLX_TENSOR_FROZEN)) && !(step_flags & RLX_STEP_ZERO_GRADS)) {
+            update_tile_paired<LANES, SP, NTL, CLIP>(r, off, lane, h, dev_params, norm);
+            return;
+        }
+    }
     const int e0 = lane * E;
     const int64_t i0 = off + e0;
     const bool zero_grads = (step_flags & RLX_STEP_ZERO_GRADS) != 0;
@@ -372,7 +431,7 @@ __device__ __forceinline__ void update_tile(const ChunkRec& r, int64_t off, int6
         // the same split costs 1-4 %, so the plain update issues all four loads at once.
         // The host launches the PH = 1 form of the kernel only for such steps, so that the plain update keeps
         // its straight-line code (a run-time test here cost it 2 %).
-        if constexpr (PH == 0) {
+        if constexpr (PH != 1) {
             load_g(); load_mv(); load_w();
         } else {
             if (has_master || zero_grads) { load_g(); load_w(); wait_for_memory(); load_mv(); }
@@ -1222,7 +1281,7 @@ struct Tuning {
                                             // has at most 8,192 workgroups, 2 = that up to 256 workgroups (default)
 } g_tuning;
 
-constexpr int kNumUpdateVariants = 17;
+constexpr int kNumUpdateVariants = 18;
 constexpr int kNumConvertVariants = 4;
 constexpr int64_t kMaxTilesPerLaunch = 1 << 23;   // workgroups per launch; times 256 lanes stays below 2^32
 constexpr int64_t kMaxNormGrid = 1 << 22;
@@ -1434,6 +1493,8 @@ const char* const kVariantNames[kNumUpdateVariants] = {
     "adamw_persistent_kernel<8,4,1,true>",     // 14: the persistent form with those
     "adamw_rounds_kernel<2,128,2,1>",          // 15: the shipped accesses, two 256-element sub-tiles per workgroup
     "adamw_rounds_kernel<2,128,4,1>",          // 16: four sub-tiles (chunks of 1,024 elements and more)
+    "adamw_tile_kernel<2,128,1,*,1,2>",        // 17: the shipped tile with lane pairs sharing 128-bit accesses: half the
+                                               //     memory instructions (whole aligned tiles of plain FP16 tensors)
 };
 
 // any_master: some tensor of the launch has an FP32 master copy.  Such launches, and those that clear the
@@ -1470,6 +1531,7 @@ int launch_update(const ChunkRec* recs, const ChunkRec& single, int64_t single_n
     case 14: if constexpr (!SINGLE) e = launch_persistent<1, true>(recs, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
     case 15: if constexpr (!SINGLE) e = launch_rounds<2, 128, 2>(recs, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
     case 16: if constexpr (!SINGLE) e = launch_rounds<2, 128, 4>(recs, n, chunk_log2, h, dev_params, norm, step_flags, s); break;
+    case 17: RLX_V(2, 128, 1, SINGLE, 1, 2); break;
     }
 #undef RLX_V
     if (e != hipSuccess) return hip_fail(e, "update kernel launch");

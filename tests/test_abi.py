@@ -135,8 +135,8 @@ def test_tuning_keys(B):
     with pytest.raises(B.RlxError):
         B.set_tuning("norm_keep_mb", 4097)
     # every update variant has a kernel name; the default names the shipped tile shape
-    names = [B.update_variant_name(v) for v in range(17)]
-    assert all(names) and len(set(names)) == 17 and B.update_variant_name(17) == ""
+    names = [B.update_variant_name(v) for v in range(18)]
+    assert all(names) and len(set(names)) == 18 and B.update_variant_name(18) == ""
     assert names[0].startswith("adamw_tile_kernel<2,128,1,") and B.update_variant_name() == names[0]
     assert "persistent" in names[11] and "chunk" in names[12]
 

@@ -290,7 +290,8 @@ def test_ragged_list_equals_flat_tensor(O, L, host, B, torch_gpu):
 def test_every_tile_shape_and_chunk_size_gives_the_same_bits(L, host, B, torch_gpu, master, zero_grads):
     """Every compiled form of the update kernel (tile shapes, XCD swizzle, store policy, the two forms that
     issue their loads and stores at once or two at a time, and the 128-bit-access forms: one wavefront per tile,
-    a persistent grid striding over the tiles, one workgroup walking a chunk) gives the same bits, with and
+    a persistent grid striding over the tiles, one workgroup walking a chunk, lane pairs sharing 128-bit accesses)
+    gives the same bits, with and
     without a master copy and gradient clearing (which select between the first two forms by default)."""
     torch = torch_gpu
     specs = [L.TensorSpec("a", 70_001, L.DTYPE_F16, 0, 0), L.TensorSpec("b", 2049, L.DTYPE_F32, 0, 0),
@@ -300,7 +301,7 @@ def test_every_tile_shape_and_chunk_size_gives_the_same_bits(L, host, B, torch_g
         for variant, chunk in [(0, 8192), (1, 8192), (2, 2048), (3, 512), (4, 512), (5, 65536), (6, 1024),
                                (7, 2048), (8, 8192), (9, 4096), (10, 512), (10, 8192), (11, 512), (11, 2048),
                                (11, 65536), (12, 512), (12, 8192), (13, 2048), (14, 8192), (15, 512), (15, 8192),
-                               (16, 512), (16, 1024), (16, 8192)]:
+                               (16, 512), (16, 1024), (16, 8192), (17, 512), (17, 2048), (17, 8192)]:
             B.set_tuning("update_variant", variant)
             st = host.ParamStore(specs, master=master)
             st.fill("p", 1, 0.0, 0.02)
