@@ -562,7 +562,8 @@ def test_scheduled_steps_replay_without_the_host(O, L, host, B, torch_gpu):
     assert opt.plan.schedule_position() == (0, 1) and opt.plan.schedule_overrun() == 0
 
 
-def test_one_recorded_step_replays_through_three_uploaded_windows(O, L, host, B, torch_gpu):
+@pytest.mark.parametrize("norm_fused", [2, 0])
+def test_one_recorded_step_replays_through_three_uploaded_windows(O, L, host, B, torch_gpu, norm_fused, request):
     """The reference sets a new learning rate from its scheduler before every step of the whole run
     (include/training/trainer.h:193-194, optimizer.h:120-122).  Here: norm + fused-clip scheduled update recorded
     ONCE as a HIP graph after the first upload, then replayed through window 1 (3 steps), a LONGER window 2
@@ -571,6 +572,8 @@ def test_one_recorded_step_replays_through_three_uploaded_windows(O, L, host, B,
     and the bias corrections of its step number; the position is right after every step and never passes the
     table's length; no step overruns its table."""
     torch = torch_gpu
+    B.set_tuning("norm_fused", norm_fused)       # the norm's sum recorded as the tail of its launch, or as a second launch
+    request.addfinalizer(lambda: B.set_tuning("norm_fused", 2))
     specs = L.qwen3_tensor_list(MINI, norm_dtype=L.DTYPE_F32, reference_decay_groups=True)
     st = host.ParamStore(specs)
     st.fill("p", 1, 0.0, 0.02)
